@@ -68,10 +68,21 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // sequence's first tiles almost never happens.  NEG_MC is -m * c, kept beside m.  VOTE = false
 // compares the lanes in every tile, without a branch: the kernel for decoded tokens is bound
 // by its loads, and a branch in its loop costs it more than the comparisons.
+// A cap on the scores, s <- cap * tanh(s / cap), is applied to the raw scores in their own units (cap_raw = cap /
+// scale, so that the factor of the softmax that follows still turns them into scaled ones), before the masks: tanh
+// of a masked score would be finite.  tanh(x) = 1 - 2 / (exp(2x) + 1): one v_exp_f32 and one v_rcp_f32.
+__device__ __forceinline__ float tanh_of(float x) {
+  const float e = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);  // exp(2x); inf for large x, whose quotient is 0
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+
 #define MAXIMUM(a, b) __builtin_elementwise_maximum(a, b)
 #define SOFTMAX_TILE(VOTE, ST0, ST1, NEED_MASK, OK_EXPR, M_RUN, NEG_MC, L_RUN, ALPHA, PF)                    \
   {                                                                                                          \
     float rv[8] = {ST0[0], ST0[1], ST0[2], ST0[3], ST1[0], ST1[1], ST1[2], ST1[3]};                          \
+    if (cap_raw > 0.f) {                                                                                     \
+      _Pragma("unroll") for (int e = 0; e < 8; ++e) rv[e] = cap_raw * tanh_of(rv[e] * inv_cap_raw);          \
+    }                                                                                                        \
     if (NEED_MASK) {                                                                                         \
       _Pragma("unroll") for (int e = 0; e < 8; ++e) {                                                        \
         const int key = kt + 8 * j + e;                                                                      \
@@ -149,7 +160,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
                       const bf16_t* __restrict__ cache, const int* __restrict__ block_table, int table_width,
                       const int* __restrict__ cu_q, const int* __restrict__ kv_len, const int* __restrict__ work,
                       int n_work, float* __restrict__ partial, int n_q_heads, int n_kv_heads, int page_size,
-                      int page_shift, int num_pages, int window_left, float scale_log2e, const float* __restrict__ sink) {
+                      int page_shift, int num_pages, int window_left, int chunk, float scale_log2e, float cap_raw,
+                      const float* __restrict__ sink) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int id = blockIdx.x;  // (item, key/value head): the same for the whole block
@@ -179,7 +191,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
   const int ti = row_valid ? r / group : 0;
   const int hq = g * group + (row_valid ? r - ti * group : 0);
   const int row_end = n_old + ti;  // last key the row may read
-  const int row_start = window_left >= 0 ? max(0, row_end - window_left) : 0;
+  const int row_start = chunk > 0 ? row_end - row_end % chunk : (window_left >= 0 ? max(0, row_end - window_left) : 0);
   // the span of keys that any row of the item reads (uniform): outside it values may be anything
   // (pages given back, slots never written) and are zeroed before use
   int lo_any = row_valid ? row_start : 0x7fffffff, hi_any = row_valid ? row_end : -1;
@@ -213,6 +225,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __res
   float4v acc[D_TILES];
   const float neg_inf = -__builtin_inff();
   const float lazy_raw = 8.0f / scale_log2e;  // 8 binary orders, in units of the raw scores
+  const float inv_cap_raw = cap_raw > 0.f ? 1.0f / cap_raw : 0.f;
 #pragma unroll
   for (int dt = 0; dt < D_TILES; ++dt) acc[dt] = (float4v){0.f, 0.f, 0.f, 0.f};
   float m_run = neg_inf, neg_mc_run = 0.f;
@@ -453,7 +466,8 @@ attention_lds_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __rest
                      const bf16_t* __restrict__ cache, const int* __restrict__ block_table, int table_width,
                      const int* __restrict__ cu_q, const int* __restrict__ kv_len, const int* __restrict__ work,
                      float* __restrict__ partial, int n_kv_heads_grid, int n_q_heads, int n_kv_heads, int page_size,
-                     int page_shift, int num_pages, int window_left, float scale_log2e, const float* __restrict__ sink) {
+                     int page_shift, int num_pages, int window_left, int chunk, float scale_log2e, float cap_raw,
+                      const float* __restrict__ sink) {
   constexpr bool FAST = MODE != LDS_PLAIN;
   constexpr int DMA_AHEAD = DMA_BUFFERS - 1;
   __shared__ __attribute__((aligned(16))) bf16_t lds_k[MODE == LDS_DMA ? 1 : 2][MODE == LDS_DMA ? 8 : 32 * LDS_K_STRIDE];
@@ -489,6 +503,7 @@ attention_lds_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __rest
   float m_run[LDS_RT], neg_mc_run[LDS_RT], l_run[LDS_RT];
   const float neg_inf = -__builtin_inff();
   const float lazy_raw = 8.0f / scale_log2e;  // 8 binary orders, in units of the raw scores
+  const float inv_cap_raw = cap_raw > 0.f ? 1.0f / cap_raw : 0.f;
 #pragma unroll
   for (int rt = 0; rt < LDS_RT; ++rt) {
     const int r = w[1] + 16 * (LDS_RT * wave + rt) + n;
@@ -496,7 +511,7 @@ attention_lds_kernel(const bf16_t* __restrict__ q, long q_stride, bf16_t* __rest
     ti[rt] = row_valid[rt] ? r / group : 0;
     hq[rt] = g * group + (row_valid[rt] ? r - ti[rt] * group : 0);
     row_end[rt] = n_old + ti[rt];
-    row_start[rt] = window_left >= 0 ? max(0, row_end[rt] - window_left) : 0;
+    row_start[rt] = chunk > 0 ? row_end[rt] - row_end[rt] % chunk : (window_left >= 0 ? max(0, row_end[rt] - window_left) : 0);
     const bf16_t* qrow = q + (size_t)(q0 + ti[rt]) * q_stride + (size_t)hq[rt] * HEAD_DIM;
 #pragma unroll
     for (int s = 0; s < K32_STEPS; ++s) {
@@ -985,8 +1000,12 @@ extern "C" int cwm_attention_mfma(const void* q, long q_stride, void* out, long 
                                   const int* work, int n_work, int work_keys, const int* work_wide, int n_work_wide, int wide_tiles,
                                   int wide_three_blocks, const int* merge,
                                   int n_merge, int n_merge_mid, int n_merge_few, float* partial, int n_q_heads, int n_kv_heads, int head_dim,
-                                  int page_size, int num_pages, int window_left, float scale, const float* sink,
-                                  hipStream_t stream) {
+                                  int page_size, int num_pages, int window_left, int chunk, float scale, float softcap,
+                                  const float* sink, hipStream_t stream) {
+  // `chunk` > 0: instead of a window, a query reads the keys of its own block of that many positions (counted from 0)
+  // up to itself; `softcap` > 0: scaled scores are capped, s <- softcap * tanh(s / softcap), before the softmax
+  CWM_REQUIRE(chunk >= 0 && softcap >= 0.f && scale > 0.f, "attention_mfma: a block of keys and a cap cannot be negative, the scale is positive");
+  const float cap_raw = softcap > 0.f ? softcap / scale : 0.f;
   // `work`: items of one 16-row tile (may be split over chunks of keys), one wavefront each;
   // `work_wide`: items of 4 * LDS_RT row tiles, one block each with keys and values in LDS
   CWM_REQUIRE(head_dim == HEAD_DIM, "attention_mfma: this library is built for head_dim %d, not %d", HEAD_DIM, head_dim);
@@ -1015,7 +1034,7 @@ extern "C" int cwm_attention_mfma(const void* q, long q_stride, void* out, long 
   hipLaunchKernelGGL((attention_mfma_kernel<PAGE32>), dim3((unsigned)blocks), dim3(256), 0, stream, (const bf16_t*)q,     \
                      q_stride, (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table, table_width, cu_q, kv_len,   \
                      work, n_work, partial, n_q_heads, n_kv_heads, page_size, page_shift, num_pages, window_left,        \
-                     scale_log2e, sink)
+                     chunk, scale_log2e, cap_raw, sink)
     if (page_size % 32 == 0)
       CWM_LAUNCH_TEAM(true);
     else
@@ -1031,7 +1050,7 @@ extern "C" int cwm_attention_mfma(const void* q, long q_stride, void* out, long 
   hipLaunchKernelGGL((attention_lds_kernel<MODE, BUFFERS, MIN_BLOCKS>), dim3((unsigned)blocks), dim3(256), 0, stream,     \
                      (const bf16_t*)q, q_stride,                                                                          \
                      (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table, table_width, cu_q, kv_len, work_wide,   \
-                     partial, n_kv_heads, n_q_heads, n_kv_heads, page_size, page_shift, num_pages, window_left, scale_log2e, sink)
+                     partial, n_kv_heads, n_q_heads, n_kv_heads, page_size, page_shift, num_pages, window_left, chunk, scale_log2e, cap_raw, sink)
     // tiles of 32 keys that never straddle a page, and shares of a tile that divide evenly over the block
     if (page_size % 32 == 0 && LDS_K_CHUNKS % 256 == 0 && LDS_V_CHUNKS % 256 == 0) {
 #if DMA_HEAD_DIM_OK

@@ -7,7 +7,9 @@
 // Formula (cwm/fastgen/forward.py:638-655): query at absolute position p of its
 // sequence reads keys j with max(0, p - window_left) <= j <= p (window_left < 0:
 // from 0); s_j = (q . k_j) * scale; o = sum_j softmax(s)_j v_j; query head h uses
-// key/value head h / (n_q_heads / n_kv_heads).
+// key/value head h / (n_q_heads / n_kv_heads).  Two options beside it: `chunk` > 0 replaces the window by blocks
+// of that many positions counted from 0 (the query at p reads the keys of its own block up to p), and `softcap` > 0
+// caps the scaled score, s_j <- softcap * tanh(s_j / softcap), before the softmax.
 //
 // One block of four wavefronts per (token, key/value head, up to 8 of its query heads,
 // segment of the keys): a key and a value are loaded once and used for all the block's
@@ -56,6 +58,12 @@ __device__ __forceinline__ int segments_of(int n_keys, int& seg_len) {
   return n_seg;
 }
 
+// the first key that the query at position p reads
+__device__ __forceinline__ int first_key_of(int p, int window_left, int chunk) {
+  if (chunk > 0) return p - p % chunk;
+  return window_left >= 0 ? max(0, p - window_left) : 0;
+}
+
 // partial result of (token, query head, segment): [head_dim] unnormalised output, then maximum and sum
 #define PARTIAL_STRIDE(hd) ((hd) + 2)
 
@@ -67,7 +75,7 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
                         const T* __restrict__ cache, const int* __restrict__ block_table, int table_width,
                         const int* __restrict__ positions, const int* __restrict__ seq_of_token, float* __restrict__ partial,
                         int n_q_heads, int n_kv_heads, int head_groups, int head_dim, int page_size, int num_pages,
-                        int window_left, float scale, const float* __restrict__ sink) {
+                        int window_left, int chunk, float scale, float softcap, const float* __restrict__ sink) {
   __shared__ __attribute__((aligned(16))) float qs[HEADS][D_REGS * CWM_WAVE];
   // probabilities of a chunk, key jj at [in0 + jj] (in0: the first key's place in its block of 8 values), so that the
   // eight of a block lie at a multiple of 8
@@ -89,7 +97,7 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
   const int nh = min(SIMPLE_HEADS, group - hg * SIMPLE_HEADS);  // and how many it serves
   const int p = positions[t];
   const int b = seq_of_token[t];
-  const int start = window_left >= 0 ? max(0, p - window_left) : 0;
+  const int start = first_key_of(p, window_left, chunk);
   int seg_len;
   const int n_seg = segments_of(p - start + 1, seg_len);
   if (seg >= n_seg) return;
@@ -194,7 +202,10 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
           }
         }
 #pragma unroll
-        for (int h = 0; h < HEADS; ++h) s[h] = dot[h] * scale;
+        for (int h = 0; h < HEADS; ++h) {
+          s[h] = dot[h] * scale;
+          if (softcap > 0.f) s[h] = softcap * tanhf(s[h] / softcap);
+        }
         // values: blocks of v_block keys, [slot / v_block][dim][slot % v_block]
         vo = (long long)((size_t)page * 2 * plane + plane + (size_t)g * head_dim * page_size +
                          (size_t)(slot / v_block) * head_dim * v_block + slot % v_block);
@@ -346,13 +357,13 @@ attention_simple_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ 
 template <typename T>
 __global__ void __launch_bounds__(CWM_WAVE)
 attention_simple_join_kernel(T* __restrict__ out, long out_stride, const float* __restrict__ partial,
-                             const int* __restrict__ positions, int n_q_heads, int head_dim, int window_left,
+                             const int* __restrict__ positions, int n_q_heads, int head_dim, int window_left, int chunk,
                              int max_segments, const float* __restrict__ sink) {
   const int t = blockIdx.x / n_q_heads;
   const int h = blockIdx.x - t * n_q_heads;
   const int lane = threadIdx.x;
   const int p = positions[t];
-  const int start = window_left >= 0 ? max(0, p - window_left) : 0;
+  const int start = first_key_of(p, window_left, chunk);
   int seg_len;
   const int n_seg = segments_of(p - start + 1, seg_len);
   if (n_seg <= 1 || n_seg > max_segments) return;  // more than the launch had room for: the rows are NaN already
@@ -392,8 +403,9 @@ attention_simple_join_kernel(T* __restrict__ out, long out_stride, const float* 
 extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, long out_stride, const void* cache,
                                     int dtype, const int* block_table, int table_width, const int* positions,
                                     const int* seq_of_token, int n_tokens, int n_q_heads, int n_kv_heads,
-                                    int head_dim, int page_size, int num_pages, int window_left, float scale,
-                                    int max_keys, float* partial, const float* sink, hipStream_t stream) {
+                                    int head_dim, int page_size, int num_pages, int window_left, int chunk, float scale,
+                                    float softcap, int max_keys, float* partial, const float* sink, hipStream_t stream) {
+  CWM_REQUIRE(chunk >= 0 && softcap >= 0.f, "attention: a block of keys and a cap on the scores cannot be negative");
   CWM_REQUIRE(n_tokens >= 0, "attention: negative token count");
   CWM_REQUIRE(head_dim > 0 && head_dim <= SIMPLE_MAX_HEAD_DIM, "attention: head_dim %d is outside 1..%d", head_dim,
               SIMPLE_MAX_HEAD_DIM);
@@ -421,7 +433,7 @@ extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, lon
   hipLaunchKernelGGL((attention_simple_kernel<float, HEADS, D_REGS>), grid, dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream,     \
                      (const float*)q, q_stride, (float*)out, out_stride, (const float*)cache, block_table, table_width,   \
                      positions, seq_of_token, partial, n_q_heads, n_kv_heads, head_groups, head_dim, page_size, num_pages, \
-                     window_left, scale, sink)
+                     window_left, chunk, scale, softcap, sink)
 #define CWM_LAUNCH_SIMPLE_HEADS(D_REGS)   \
   do {                                    \
     if (heads <= 2)                       \
@@ -443,15 +455,15 @@ extern "C" int cwm_attention_simple(const void* q, long q_stride, void* out, lon
 #undef CWM_LAUNCH_SIMPLE
     if (max_segments > 1)
       hipLaunchKernelGGL(attention_simple_join_kernel<float>, dim3((unsigned)join_blocks), dim3(CWM_WAVE), 0, stream,
-                         (float*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left, max_segments, sink);
+                         (float*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left, chunk, max_segments, sink);
   } else if (dtype == CWM_BF16) {
     hipLaunchKernelGGL((attention_simple_kernel<bf16_t, SIMPLE_HEADS, SIMPLE_D_REGS>), grid, dim3(SIMPLE_WAVES * CWM_WAVE), 0, stream, (const bf16_t*)q,
                        q_stride, (bf16_t*)out, out_stride, (const bf16_t*)cache, block_table, table_width, positions,
                        seq_of_token, partial, n_q_heads, n_kv_heads, head_groups, head_dim, page_size, num_pages, window_left,
-                       scale, sink);
+                       chunk, scale, softcap, sink);
     if (max_segments > 1)
       hipLaunchKernelGGL(attention_simple_join_kernel<bf16_t>, dim3((unsigned)join_blocks), dim3(CWM_WAVE), 0, stream,
-                         (bf16_t*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left, max_segments, sink);
+                         (bf16_t*)out, out_stride, (const float*)partial, positions, n_q_heads, head_dim, window_left, chunk, max_segments, sink);
   } else {
     return cwm_fail("attention: unknown dtype %d", dtype);
   }

@@ -509,3 +509,159 @@ extern "C" int cwm_qk_norm_rope_write(const void* src, int src_dtype, long src_s
 #undef CWM_NORM_ROPE_V
   return cwm_launch_status("qk_norm_rope_write");
 }
+
+// ---- projection rows -> bias -> norm of every head -> rotation -> (values mixed with another layer's) -> cache -- //
+// A token's row of the joined projection is [q: Hq * qk_dim | k: Hkv * qk_dim | v: Hkv * v_dim | ...] (type TS, or
+// float32 partial sums of a split K, added in order), to which `bias` (float32, one value a column of q, k and v) is
+// added.  Every query head and every key head is divided by its own root mean square (eps inside the root) and
+// multiplied by a weight of qk_dim values that all heads share, where a weight is given; then rotated by
+// position * inv_freq[pair] (adjacent pairs; a frequency of 0 leaves its pair alone).  Values: where `v_other` is
+// given, v <- (1 - mix) v + mix v_other, with `mix` one float32 on the device and v_other [T][Hkv * v_dim] the
+// values that another layer made of the same tokens; `v_keep`, where given, receives this layer's values as they go
+// into the cache, [T][Hkv * v_dim].  Heads are laid out with `head_dim` elements as in the kernel above.  All
+// arithmetic float32.  A wavefront a head: the lanes hold the head's pairs, so a head's sum of squares is one
+// reduction over the lanes; the blocks of a token (gridDim.y of them) share its heads.
+template <typename TS, typename TO>
+__global__ void __launch_bounds__(256)
+head_norm_rope_write_kernel(const TS* __restrict__ src, long src_stride, int n_partials, long partial_stride,
+                            const float* __restrict__ bias, TO* __restrict__ q_out, const float* __restrict__ q_weight,
+                            const float* __restrict__ k_weight, float eps, const int* __restrict__ positions,
+                            const int* __restrict__ seq_of_token, const float* __restrict__ inv_freq, TO* __restrict__ cache,
+                            const int* __restrict__ block_table, int table_width, int page_size, int num_pages, int n_q_heads,
+                            int n_kv_heads, int qk_dim, int v_dim, int head_dim, const TO* __restrict__ v_other,
+                            long v_other_stride, const float* __restrict__ v_mix, TO* __restrict__ v_keep) {
+  __shared__ __attribute__((aligned(16))) float cs[NORM_ROPE_MAX_HEAD];  // cos, sin of each pair
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int half = head_dim / 2;
+  const int lane = threadIdx.x & (CWM_WAVE - 1);
+  const int wave = threadIdx.x / CWM_WAVE;
+  const int q_width = n_q_heads * qk_dim, k_width = n_kv_heads * qk_dim;
+  const TS* srow = src + (size_t)t * src_stride;
+  auto value = [&](int e) {
+    float v = 0.f;
+    for (int p = 0; p < n_partials; ++p) v += Elem<TS>::load(srow + (size_t)p * partial_stride + e);
+    return bias ? v + bias[e] : v;
+  };
+  TO* kdst = nullptr;
+  TO* vdst = nullptr;
+  int slot = 0;
+  if (cache) {
+    const int seq = seq_of_token[t];
+    const int lp = pos / page_size;
+    slot = pos - lp * page_size;
+    const int page = (lp >= 0 && lp < table_width) ? block_table[(size_t)seq * table_width + lp] : -1;
+    if (page >= 0 && page < num_pages) {
+      const size_t plane = (size_t)n_kv_heads * page_size * head_dim;
+      kdst = cache + (size_t)page * 2 * plane;
+      vdst = kdst + plane;
+    }
+  }
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    float c = 1.f, s = 0.f;
+    const float f = inv_freq ? inv_freq[i] : 0.f;
+    if (f != 0.f) sincosf((float)pos * f, &s, &c);
+    cs[2 * i] = c;
+    cs[2 * i + 1] = s;
+  }
+  __syncthreads();
+  const int n_heads = n_q_heads + (cache ? n_kv_heads : 0);
+  const int waves = blockDim.x / CWM_WAVE;
+  for (int hh = blockIdx.y * waves + wave; hh < n_heads; hh += gridDim.y * waves) {
+    const bool is_key = hh >= n_q_heads;
+    const int head = is_key ? hh - n_q_heads : hh;
+    const int base = (is_key ? q_width : 0) + head * qk_dim;
+    const float* weight = is_key ? k_weight : q_weight;
+    // pairs lane, lane + 64 of the head
+    float re[2], im[2];
+    float ss = 0.f;
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int i = lane + CWM_WAVE * r;
+      re[r] = (i < half && 2 * i < qk_dim) ? value(base + 2 * i) : 0.f;
+      im[r] = (i < half && 2 * i + 1 < qk_dim) ? value(base + 2 * i + 1) : 0.f;
+      ss += re[r] * re[r] + im[r] * im[r];
+    }
+    float rstd = 1.f;
+    if (weight) rstd = 1.0f / sqrtf(wave_sum(ss) / (float)qk_dim + eps);
+    TO* dst = nullptr;
+    if (!is_key)
+      dst = q_out + ((size_t)t * n_q_heads + head) * head_dim;
+    else if (kdst)
+      dst = kdst + ((size_t)head * page_size + slot) * head_dim;
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int i = lane + CWM_WAVE * r;
+      if (i < half && dst) {
+        float a = re[r], b = im[r];
+        if (weight) {
+          a *= rstd * (2 * i < qk_dim ? weight[2 * i] : 0.f);
+          b *= rstd * (2 * i + 1 < qk_dim ? weight[2 * i + 1] : 0.f);
+        }
+        const float c = cs[2 * i], s = cs[2 * i + 1];
+        Elem<TO>::store(dst + 2 * i, a * c - b * s);
+        Elem<TO>::store(dst + 2 * i + 1, b * c + a * s);
+      }
+    }
+  }
+  if (vdst || v_keep) {
+    const int v_block = (page_size % 8 == 0) ? 8 : page_size;
+    const int v_base = q_width + k_width;
+    const float mix = (v_other && v_mix) ? *v_mix : 0.f;
+    for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < n_kv_heads * head_dim; e += gridDim.y * blockDim.x) {
+      const int head = e / head_dim, d = e - head * head_dim;
+      float v = 0.f;
+      if (d < v_dim) {
+        v = value(v_base + head * v_dim + d);
+        if (v_other) v = (1.0f - mix) * v + mix * Elem<TO>::load(v_other + (size_t)t * v_other_stride + head * v_dim + d);
+        if (v_keep) Elem<TO>::store(v_keep + ((size_t)t * n_kv_heads + head) * v_dim + d, v);
+      }
+      if (vdst)
+        Elem<TO>::store(vdst + (size_t)head * head_dim * page_size + ((size_t)(slot / v_block) * head_dim + d) * v_block + slot % v_block, v);
+    }
+  }
+}
+
+// src: [n_tokens][src_stride] of src_dtype (the row may go on beyond q, k and v), or n_partials float32 slabs
+// partial_stride apart.  bias: float32 [(Hq + Hkv) * qk_dim + Hkv * v_dim] or null.  q_weight, k_weight: float32
+// [qk_dim] or null.  inv_freq: float32 [head_dim / 2] or null.  v_other ([n_tokens][v_other_stride], the cache's type)
+// with v_mix (one float32 on the device): both or neither.  v_keep: [n_tokens][Hkv * v_dim] of the cache's type, or null.
+extern "C" int cwm_head_norm_rope_write(const void* src, int src_dtype, long src_stride, int n_partials, long partial_stride,
+                                        const float* bias, void* q_out, int out_dtype, const float* q_weight, const float* k_weight,
+                                        float eps, const int* positions, const int* seq_of_token, const float* inv_freq, void* cache,
+                                        const int* block_table, int table_width, int page_size, int num_pages, int n_tokens,
+                                        int n_q_heads, int n_kv_heads, int qk_dim, int v_dim, int head_dim, const void* v_other,
+                                        long v_other_stride, const float* v_mix, void* v_keep, hipStream_t stream) {
+  CWM_REQUIRE(n_tokens >= 0 && n_partials >= 1, "head_norm_rope_write: bad sizes");
+  CWM_REQUIRE(n_partials == 1 || src_dtype == CWM_F32, "head_norm_rope_write: partial sums must be float32");
+  CWM_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= NORM_ROPE_MAX_HEAD,
+              "head_norm_rope_write: head_dim %d must be even and at most %d", head_dim, NORM_ROPE_MAX_HEAD);
+  CWM_REQUIRE(qk_dim >= 1 && v_dim >= 1 && qk_dim <= head_dim && v_dim <= head_dim,
+              "head_norm_rope_write: heads of %d (queries, keys) and %d (values) do not fit the cached head of %d", qk_dim, v_dim, head_dim);
+  CWM_REQUIRE(n_q_heads > 0 && n_kv_heads > 0, "head_norm_rope_write: no heads");
+  CWM_REQUIRE(src && q_out && positions, "head_norm_rope_write: arguments missing");
+  CWM_REQUIRE(eps > 0.f || (!q_weight && !k_weight), "head_norm_rope_write: eps must be positive");
+  CWM_REQUIRE((v_other == nullptr) == (v_mix == nullptr), "head_norm_rope_write: other values and their weight come together");
+  if (cache) {
+    CWM_REQUIRE(block_table && seq_of_token, "head_norm_rope_write: a cache write needs a block table");
+    CWM_REQUIRE(page_size > 0 && num_pages > 0 && table_width > 0, "head_norm_rope_write: bad cache geometry");
+  }
+  if (n_tokens == 0) return 0;
+  const int key = (src_dtype << 1) | out_dtype;
+  // few tokens: several blocks a token, so that a decode step's rows are not left to as many blocks
+  const int heads = n_q_heads + n_kv_heads;
+  const int gy = n_tokens >= 512 ? 1 : (heads <= 4 ? 1 : (heads < 32 ? (heads + 3) / 4 : 8));
+#define CWM_HEAD_NORM_ROPE(TS, TO)                                                                                         \
+  hipLaunchKernelGGL((head_norm_rope_write_kernel<TS, TO>), dim3(n_tokens, gy), dim3(256), 0, stream, (const TS*)src,       \
+                     src_stride, n_partials, partial_stride, bias, (TO*)q_out, q_weight, k_weight, eps, positions,         \
+                     seq_of_token, inv_freq, (TO*)cache, block_table, table_width, page_size, num_pages, n_q_heads,        \
+                     n_kv_heads, qk_dim, v_dim, head_dim, (const TO*)v_other, v_other_stride, v_mix, (TO*)v_keep)
+  switch (key) {
+    case 0: CWM_HEAD_NORM_ROPE(float, float); break;
+    case 1: CWM_HEAD_NORM_ROPE(float, bf16_t); break;
+    case 3: CWM_HEAD_NORM_ROPE(bf16_t, bf16_t); break;
+    default: return cwm_fail("head_norm_rope_write: source type %d with cache type %d is not built", src_dtype, out_dtype);
+  }
+#undef CWM_HEAD_NORM_ROPE
+  return cwm_launch_status("head_norm_rope_write");
+}

@@ -807,6 +807,15 @@ def _check_sink(sink: Optional[torch.Tensor], n_q: int) -> None:
         raise KernelError(f"the sinks must be a contiguous float32 [{n_q}] tensor, one a query head")
 
 
+def _check_mask(window: Optional[int], chunk: Optional[int], softcap: Optional[float]) -> None:
+    if window is not None and window < 1:
+        raise KernelError("a window holds at least the query's own key")
+    if chunk is not None and (chunk < 1 or window is not None):
+        raise KernelError("a block of keys holds at least one position, and comes instead of a window")
+    if softcap is not None and not softcap > 0:
+        raise KernelError("a cap on the scores must be positive")
+
+
 def paged_attention_simple(
     q: torch.Tensor,
     cache: torch.Tensor,
@@ -817,14 +826,19 @@ def paged_attention_simple(
     scale: float,
     max_keys: Optional[int] = None,
     sink: Optional[torch.Tensor] = None,
+    softcap: Optional[float] = None,
+    chunk: Optional[int] = None,
 ) -> torch.Tensor:
     """Causal attention of `q` [T, Hq, hd] over the paged cache by the plain kernel:
     float32 arithmetic, a key/value head's query heads sharing its keys and values, long
     key ranges cut into segments that a second kernel joins.  `window`: keys read per
     query, own included (None: all).  `max_keys`: the most keys any token reads (default:
     from the largest position, which costs a copy to the host).  `sink`: float32 [Hq], a term exp(sink) that
-    each head's softmax denominator holds beside its keys (no key, no value, not scaled).  Returns [T, Hq * hd]."""
+    each head's softmax denominator holds beside its keys (no key, no value, not scaled).  `softcap`: scaled scores
+    become softcap * tanh(score / softcap) before the softmax.  `chunk` (instead of a window): a query reads the keys of
+    its own block of that many positions, counted from 0, up to itself.  Returns [T, Hq * hd]."""
     _need_gpu(q, cache, block_table, positions, seq_of_token, sink)
+    _check_mask(window, chunk, softcap)
     _check_sink(sink, q.shape[1] if q.dim() == 3 else 0)
     if q.dim() != 3 or q.stride(2) != 1 or q.stride(1) != q.shape[2]:
         raise KernelError("q must be [T, Hq, hd] with contiguous heads")
@@ -839,14 +853,12 @@ def paged_attention_simple(
     _i32(seq_of_token, "seq_of_token")
     if positions.numel() != n_tokens or seq_of_token.numel() != n_tokens or block_table.dim() != 2:
         raise KernelError("positions and seq_of_token must be [T], block_table [B, W]")
-    if window is not None and window < 1:
-        raise KernelError("a window holds at least the query's own key")
     out = torch.empty((n_tokens, n_q * hd), dtype=q.dtype, device=q.device)
     lib = _build.load("attention_simple")
     if max_keys is None:
         max_keys = int(positions.max()) + 1 if n_tokens else 1
-    if window is not None:
-        max_keys = min(max_keys, window)
+    if window is not None or chunk is not None:
+        max_keys = min(max_keys, window if chunk is None else chunk)
     max_keys = max(1, max_keys)
     partial = None
     if max_keys > lib.cwm_attention_simple_segment_keys():
@@ -858,8 +870,8 @@ def paged_attention_simple(
             ctypes.c_int(_code(q.dtype)), _ptr(block_table), ctypes.c_int(block_table.shape[1]),
             _ptr(positions), _ptr(seq_of_token), ctypes.c_int(n_tokens), ctypes.c_int(n_q), ctypes.c_int(n_kv),
             ctypes.c_int(hd), ctypes.c_int(cache.shape[3] // hd), ctypes.c_int(cache.shape[0]),
-            ctypes.c_int(-1 if window is None else window - 1), ctypes.c_float(scale),
-            ctypes.c_int(max_keys), _ptr(partial), _ptr(sink), _stream(),
+            ctypes.c_int(-1 if window is None else window - 1), ctypes.c_int(chunk or 0), ctypes.c_float(scale),
+            ctypes.c_float(softcap or 0.0), ctypes.c_int(max_keys), _ptr(partial), _ptr(sink), _stream(),
         ),
     )
     return out
@@ -891,24 +903,24 @@ class StaticPlans:
     def __init__(self, device: torch.device, max_keys: int) -> None:
         self.device = device
         self.max_keys = max_keys  # the most keys a sequence may hold while the capture is in use
-        self.homes: dict = {}  # (group, key/value heads, window) -> (capacity, device vector, uploaded plan)
+        self.homes: dict = {}  # (group, key/value heads, window, chunk) -> (capacity, device vector, uploaded plan)
 
-    def _padded(self, batch, group: int, n_kv: int, window: Optional[int], capacity):
+    def _padded(self, batch, group: int, n_kv: int, window: Optional[int], capacity, chunk: Optional[int] = None):
         from .attention_plan import build_plan, capacity_until, pad_plan
 
         wide_cut_below = -(-2 * _compute_units(self.device) // n_kv)
         if capacity is None:
-            plan, capacity = capacity_until(batch.q_lens, batch.kv_lens, group, window, wide_cut_below, self.max_keys)
+            plan, capacity = capacity_until(batch.q_lens, batch.kv_lens, group, window, wide_cut_below, self.max_keys, chunk)
         else:
-            plan = build_plan(batch.q_lens, batch.kv_lens, group, window, wide_cut_below)
+            plan = build_plan(batch.q_lens, batch.kv_lens, group, window, wide_cut_below, chunk)
         flat = pad_plan(plan, capacity)
         return plan, capacity, flat
 
-    def plan(self, batch, group: int, n_kv: int, window: Optional[int]) -> "_UploadedPlan":
-        key = (group, n_kv, window)
+    def plan(self, batch, group: int, n_kv: int, window: Optional[int], chunk: Optional[int] = None) -> "_UploadedPlan":
+        key = (group, n_kv, window, chunk)
         home = self.homes.get(key)
         if home is None:
-            plan, capacity, flat = self._padded(batch, group, n_kv, window, None)
+            plan, capacity, flat = self._padded(batch, group, n_kv, window, None, chunk)
             if flat is None:
                 raise KernelError("this step's attention work has items that a captured step does not take")
             dev = torch.from_numpy(flat).pin_memory().to(self.device, non_blocking=True)
@@ -923,27 +935,27 @@ class StaticPlans:
 
     def refresh(self, batch) -> bool:
         """Fill every home with the lists of `batch`; False if one of them has outgrown its home."""
-        for (group, n_kv, window), (capacity, dev, _) in self.homes.items():
-            _, _, flat = self._padded(batch, group, n_kv, window, capacity)
+        for (group, n_kv, window, chunk), (capacity, dev, _) in self.homes.items():
+            _, _, flat = self._padded(batch, group, n_kv, window, capacity, chunk)
             if flat is None:
                 return False
             dev.copy_(torch.from_numpy(flat).pin_memory(), non_blocking=True)
         return True
 
 
-def _attention_plan(batch, group: int, n_kv: int, window: Optional[int], device: torch.device) -> _UploadedPlan:
-    """The step's work list for this (group size, key/value heads, window), uploaded once per step."""
+def _attention_plan(batch, group: int, n_kv: int, window: Optional[int], device: torch.device, chunk: Optional[int] = None) -> _UploadedPlan:
+    """The step's work list for this (group size, key/value heads, window or block of keys), uploaded once per step."""
     from .attention_plan import build_plan
 
     static = getattr(batch, "static", None)
     if static is not None:
-        return static.plan(batch, group, n_kv, window)
-    key = ("attention_plan", group, n_kv, window)
+        return static.plan(batch, group, n_kv, window, chunk)
+    key = ("attention_plan", group, n_kv, window, chunk)
     cached = batch.scratch.get(key)
     if cached is None:
         # a sequence whose blocks of 128 rows, over all key/value heads, would not give every compute unit two
         wide_cut_below = -(-2 * _compute_units(device) // n_kv) if device.type == "cuda" else 0
-        plan = build_plan(batch.q_lens, batch.kv_lens, group, window, wide_cut_below)
+        plan = build_plan(batch.q_lens, batch.kv_lens, group, window, wide_cut_below, chunk)
         flat = np.concatenate([plan.work.reshape(-1), plan.work_wide.reshape(-1), plan.merge.reshape(-1)]).astype(np.int32)
         host = torch.from_numpy(flat)
         if device.type == "cuda":
@@ -996,10 +1008,13 @@ def paged_attention_mfma(
     window: Optional[int],
     scale: float,
     sink: Optional[torch.Tensor] = None,
+    softcap: Optional[float] = None,
+    chunk: Optional[int] = None,
 ) -> torch.Tensor:
     """Matrix-core attention (bfloat16): prompt portions and decoded tokens in one
-    launch, long key ranges of short sequences split and merged.  `sink`: as in `paged_attention_simple`."""
+    launch, long key ranges of short sequences split and merged.  `sink`, `softcap`, `chunk`: as in `paged_attention_simple`."""
     _need_gpu(q, cache, block_table, sink)
+    _check_mask(window, chunk, softcap)
     _check_sink(sink, q.shape[1] if q.dim() == 3 else 0)
     if q.dtype != torch.bfloat16 or cache.dtype != torch.bfloat16:
         raise KernelError("the matrix-core attention kernel takes bfloat16 only")
@@ -1019,9 +1034,7 @@ def paged_attention_mfma(
     _i32(block_table, "block_table")
     if block_table.dim() != 2 or block_table.shape[0] != batch.n_seqs or n_tokens != batch.n_tokens:
         raise KernelError("block_table must be [B, W] for the batch's sequences, q [T, ...] for its tokens")
-    if window is not None and window < 1:
-        raise KernelError("a window holds at least the query's own key")
-    plan = _attention_plan(batch, n_q // n_kv, n_kv, window, q.device)
+    plan = _attention_plan(batch, n_q // n_kv, n_kv, window, q.device, chunk)
     out = torch.empty((n_tokens, n_q * hd), dtype=q.dtype, device=q.device)
     partial = None
     if plan.n_partials:
@@ -1037,8 +1050,8 @@ def paged_attention_mfma(
             ctypes.c_int(_three_blocks_a_unit(plan.n_wide * n_kv, plan.wide_shape, q.device)),
             _ptr(plan.merge), ctypes.c_int(plan.n_merge), ctypes.c_int(plan.n_merge_mid), ctypes.c_int(plan.n_merge_wide), _ptr(partial),
             ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(hd), ctypes.c_int(page_size),
-            ctypes.c_int(cache.shape[0]), ctypes.c_int(-1 if window is None else window - 1),
-            ctypes.c_float(scale), _ptr(sink), _stream(),
+            ctypes.c_int(cache.shape[0]), ctypes.c_int(-1 if window is None else window - 1), ctypes.c_int(chunk or 0),
+            ctypes.c_float(scale), ctypes.c_float(softcap or 0.0), _ptr(sink), _stream(),
         ),
     )
     return out
@@ -1052,6 +1065,8 @@ def paged_attention(
     window: Optional[int],
     scale: float,
     sink: Optional[torch.Tensor] = None,
+    softcap: Optional[float] = None,
+    chunk: Optional[int] = None,
 ) -> torch.Tensor:
     """Attention of the step's tokens over the cache.  `batch` is the step's
     `StepBatch` (positions, sequence of each token and the per-sequence lengths).
@@ -1059,10 +1074,12 @@ def paged_attention(
     matrix cores; float32, and other sizes, on the plain kernel."""
     hd = q.shape[2]
     if q.is_cuda and mfma_attention_takes(q.dtype, hd, cache.shape[3] // hd):
-        return paged_attention_mfma(q, cache, block_table, batch, window, scale, sink)
+        return paged_attention_mfma(q, cache, block_table, batch, window, scale, sink, softcap, chunk)
     static = getattr(batch, "static", None)
     max_keys = batch.max_kv_len if static is None else static.max_keys
-    return paged_attention_simple(q, cache, block_table, batch.positions, batch.seq_of_token, window, scale, max_keys=max_keys, sink=sink)
+    return paged_attention_simple(
+        q, cache, block_table, batch.positions, batch.seq_of_token, window, scale, max_keys=max_keys, sink=sink, softcap=softcap, chunk=chunk,
+    )
 
 
 # --------------------------------------------------------------------------- #
@@ -1212,11 +1229,14 @@ def measure_mfma_rate(device: torch.device, blocks: int, rounds: int, launches: 
 # --------------------------------------------------------------------------- #
 # entry points that live in modules of their own; parts reach them as `ops.<name>` like the ones above
 from .sequence import (  # noqa: E402
-    MAX_CONV_TAPS, MAX_SSM_STATE, add_rows, cast_rows, causal_conv_silu, group_rmsnorm, scan_state_elems, scan_state_pack,
+    MAX_CONV_TAPS, MAX_MEMORY_DIM, MAX_SSM_STATE, ScaledSum, add_layernorm, add_rows, cast_rows, causal_conv_silu, group_rmsnorm,
+    layernorm_limits, matrix_memory, matrix_memory_state_elems, matrix_memory_state_unpack, scan_state_elems, scan_state_pack,
     scan_state_unpack, selective_scan, sigmoid_mul, token_shift,
 )
 from .routed import (  # noqa: E402
     MAX_EXPERTS, MAX_ROUTE_TOP, ExpertGroups, GatedActivation, absorb_queries, combine_routed, expand_values, group_by_expert,
     grouped_gate_up, grouped_linear, route_top,
 )
-from .streams import ACTIVATIONS, MAX_STREAMS, RoutedSum, act_rows, embedding_streams, qk_norm_rope_write, stream_mix_norm  # noqa: E402
+from .streams import (  # noqa: E402
+    ACTIVATIONS, MAX_STREAMS, RoutedSum, act_rows, embedding_streams, head_norm_rope_write, qk_norm_rope_write, stream_mix_norm,
+)

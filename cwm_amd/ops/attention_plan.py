@@ -49,10 +49,22 @@ class AttentionPlan:
     n_merge_mid: int = 0  # how many before those have at most MERGE_MID_MAX partials; the items before them have more
 
 
+def first_keys(last_key, window: Optional[int], chunk: Optional[int]):
+    """The first key that the query at position `last_key` (a number or an array) reads: with a `window`, the
+    window - 1 keys before its own; with a `chunk`, the start of its own block of that many positions; else 0."""
+    last_key = np.asarray(last_key)
+    if chunk is not None:
+        return last_key - last_key % chunk
+    if window is not None:
+        return np.maximum(0, last_key - (window - 1))
+    return np.zeros_like(last_key)
+
+
 def build_plan(
-    q_lens: Sequence[int], kv_lens: Sequence[int], group: int, window: Optional[int], wide_cut_below: int = 0
+    q_lens: Sequence[int], kv_lens: Sequence[int], group: int, window: Optional[int], wide_cut_below: int = 0,
+    chunk: Optional[int] = None,
 ) -> AttentionPlan:
-    """`wide_cut_below`: a sequence with fewer wide items than this has their keys cut at multiples of
+    """`window` or `chunk` (at most one): which keys a query reads, see `first_keys`.  `wide_cut_below`: a sequence with fewer wide items than this has their keys cut at multiples of
     WIDE_CHUNK (its blocks alone would leave compute units idle), with fewer than an eighth of it at
     multiples of WIDE_CHUNK_FINE; the caller derives the number from the model's heads and the chip,
     so that it is the same whatever else the batch holds."""
@@ -65,7 +77,7 @@ def build_plan(
     # ---- sequences with many rows: WIDE_TILES tiles form a block that shares keys and values in LDS
     wide_seq, wide_row0, wide_lo, wide_hi, wide_n_tiles, wide_cut = [], [], [], [], [], []
     for b in np.nonzero(is_wide)[0]:
-        lo, hi, row0 = _tile_ranges(int(q[b]), int(kv[b]), int(n_tiles[b]), group, window)
+        lo, hi, row0 = _tile_ranges(int(q[b]), int(kv[b]), int(n_tiles[b]), group, window, chunk)
         n_wide = (int(n_tiles[b]) + WIDE_TILES - 1) // WIDE_TILES
         first = np.arange(n_wide) * WIDE_TILES
         last = np.minimum(first + WIDE_TILES - 1, int(n_tiles[b]) - 1)
@@ -87,16 +99,16 @@ def build_plan(
     first_tok = row0 // group
     last_tok = np.minimum(row0 + ROWS_PER_TILE - 1, n_rows[seq] - 1) // group
     hi = n_old + last_tok + 1  # exclusive
-    lo = np.zeros_like(hi) if window is None else np.maximum(0, n_old + first_tok - (window - 1))
-    chunk = chunk_keys(hi - lo)
-    c0 = lo // chunk
-    n_chunks = (hi - 1) // chunk - c0 + 1
+    lo = first_keys(n_old + first_tok, window, chunk)
+    cut = chunk_keys(hi - lo)
+    c0 = lo // cut
+    n_chunks = (hi - 1) // cut - c0 + 1
     split = n_chunks > 1
     slot0 = np.cumsum(np.where(split, n_chunks, 0)) - np.where(split, n_chunks, 0)  # first partial slot of a split tile
     item_tile = np.repeat(np.arange(tile.size), n_chunks)
     item_first = np.cumsum(n_chunks) - n_chunks
     c = np.arange(int(n_chunks.sum()), dtype=np.int64) - item_first[item_tile]  # chunk index within its tile
-    ck = chunk[item_tile]
+    ck = cut[item_tile]
     work = np.zeros((c.size, WORK_INTS), dtype=np.int32)
     work[:, 0] = seq[item_tile]
     work[:, 1] = row0[item_tile]
@@ -163,7 +175,7 @@ def build_plan(
     )
 
 
-def _tile_ranges(n_new: int, kv: int, n_tiles: int, group: int, window: Optional[int]):
+def _tile_ranges(n_new: int, kv: int, n_tiles: int, group: int, window: Optional[int], chunk: Optional[int] = None):
     """First and end key and first row of each 16-row tile of one sequence."""
     n_old = kv - n_new
     n_rows = n_new * group
@@ -171,7 +183,7 @@ def _tile_ranges(n_new: int, kv: int, n_tiles: int, group: int, window: Optional
     first_tok = row0 // group
     last_tok = np.minimum(row0 + ROWS_PER_TILE - 1, n_rows - 1) // group
     key_hi = n_old + last_tok + 1  # exclusive
-    key_lo = np.zeros_like(row0) if window is None else np.maximum(0, n_old + first_tok - (window - 1))
+    key_lo = first_keys(n_old + first_tok, window, chunk)
     return key_lo, key_hi, row0
 
 
@@ -218,22 +230,24 @@ CHUNK_RULE_ENDS = (2048, 8192, 65536)
 
 
 def capacity_until(
-    q_lens: Sequence[int], kv_lens: Sequence[int], group: int, window: Optional[int], wide_cut_below: int, max_keys: int
+    q_lens: Sequence[int], kv_lens: Sequence[int], group: int, window: Optional[int], wide_cut_below: int, max_keys: int,
+    chunk: Optional[int] = None,
 ) -> "tuple[AttentionPlan, PlanCapacity]":
     """The step's plan, and the sizes of its lists for as long as no sequence holds more than `max_keys` keys
     (every sequence growing by a token a step): the sequences as they are, all of them grown to `max_keys`, and
     grown to each length in between at which the rule for cutting the keys changes."""
-    plan = build_plan(q_lens, kv_lens, group, window, wide_cut_below)
+    plan = build_plan(q_lens, kv_lens, group, window, wide_cut_below, chunk)
     plans = [plan]
     for length in sorted({max_keys, *(n + d for n in CHUNK_RULE_ENDS for d in (0, 1) if n + d < max_keys)}):
         grown = [min(max(kv, length), max(kv, max_keys)) for kv in kv_lens]
         if grown != list(kv_lens):
-            plans.append(build_plan(q_lens, grown, group, window, wide_cut_below))
+            plans.append(build_plan(q_lens, grown, group, window, wide_cut_below, chunk))
     capacity = PlanCapacity.covering(plans)
-    if window is not None and max(max(kv_lens), max_keys) > window:
+    span = window if chunk is None else chunk
+    if span is not None and max(max(kv_lens), max_keys) > span:
         # a window's range moves over the fixed positions of the cuts: at some steps it straddles one cut more than at
         # others, whatever its length (a window shorter than a chunk is cut in two now and then).  While no sequence
-        # is longer than the window every range starts at key 0, as without a window.
+        # is longer than the window every range starts at key 0, as without a window.  A block of positions moves likewise.
         tiles = int((plan.work[:, 4] < 0).sum()) + plan.merge.shape[0]
         capacity = PlanCapacity(work=capacity.work + tiles, merge_many=capacity.merge_many, merge_mid=max(capacity.merge_mid, tiles))
     return plan, capacity

@@ -59,6 +59,8 @@ SOURCES: Dict[str, Tuple[Mapping[str, int], ...]] = {
     "state_space": ({},),
     "routed": ({},),
     "streams": ({},),
+    "layernorm": ({},),
+    "matrix_memory": ({},),
     "attention_mfma": tuple({"HEAD_DIM": hd} for hd in (16, 32, 48, 64, 80, 96, 128, 256)),
 }
 

@@ -311,3 +311,172 @@ def selective_scan(
         ),
     )
     return y
+
+
+# --------------------------------------------------------------------------- #
+class ScaledSum:
+    """A sum that has not been done yet: `terms` is a list of (tensor, factor), each tensor [T, D] (rows may lie
+    apart) or float32 partial sums [P, T, D].  The kernel that reads it next adds the terms up in their order,
+    in float32: the results of several sublayers that all join the residual at once."""
+
+    def __init__(self, terms) -> None:
+        self.terms = [(t, float(c)) for t, c in terms]
+
+    def total(self, dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        """The sum as one tensor (for readers that have no kernel of their own for it)."""
+        out = None
+        for t, c in self.terms:
+            x = (t.sum(dim=0) if t.dim() == 3 else t).to(torch.float32) * c
+            out = x if out is None else out + x
+        return out.to(dtype)
+
+
+_ln_limits: Optional[tuple] = None
+
+
+def layernorm_limits() -> tuple:
+    """(most addends, longest row) that `add_layernorm` takes, asked of the kernel library."""
+    global _ln_limits
+    if _ln_limits is None:
+        lib = _build.load("layernorm")
+        _ln_limits = (int(lib.cwm_layernorm_max_addends()), int(lib.cwm_layernorm_max_dim()))
+    return _ln_limits
+
+
+def add_layernorm(
+    h: torch.Tensor,
+    delta: Any,
+    weight: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    eps: float,
+    out_dtype: torch.dtype,
+    rows: Optional[torch.Tensor] = None,
+    weight2: Optional[torch.Tensor] = None,
+    bias2: Optional[torch.Tensor] = None,
+):
+    """`h` (float32 [T, D]) += `delta` in place, then the layer norm of its rows, (x - mean) / sqrt(var + eps) * weight
+    + bias with the variance taken about the mean, in float32.  `delta`: None, a tensor [T, D], float32 partial sums
+    [P, T, D], or a `ScaledSum` of such.  With `weight2` and `bias2` a second norm of the same rows (one mean, one
+    variance) is returned beside the first.  With `rows` (int32 [R]) only those rows are normalised and `h` is not
+    changed.  Without `weight` only the sum is done and nothing is returned."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(h, weight, bias, rows, weight2, bias2)
+    if h.dtype != torch.float32 or h.dim() != 2 or not h.is_contiguous():
+        raise KernelError("the residual stream must be a contiguous float32 [T, D] tensor")
+    n_tokens, dim = h.shape
+    max_addends, max_dim = layernorm_limits()
+    if dim > max_dim:
+        raise KernelError(f"rows of {dim} elements: the layer norm kernel takes up to {max_dim}")
+    terms = [] if delta is None else (delta.terms if isinstance(delta, ScaledSum) else [(delta, 1.0)])
+    if len(terms) > max_addends:
+        raise KernelError(f"{len(terms)} addends: the layer norm kernel takes up to {max_addends}")
+    ptrs = (ctypes.c_void_p * max(1, len(terms)))()
+    dtypes = (ctypes.c_int * max(1, len(terms)))()
+    lds = (ctypes.c_long * max(1, len(terms)))()
+    partials = (ctypes.c_int * max(1, len(terms)))()
+    strides = (ctypes.c_long * max(1, len(terms)))()
+    scales = (ctypes.c_float * max(1, len(terms)))()
+    for i, (t, c) in enumerate(terms):
+        _need_gpu(t)
+        if t.dim() == 3:
+            if t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape[1:]) != (n_tokens, dim):
+                raise KernelError(f"partial sums {tuple(t.shape)} must be contiguous float32 [P, {n_tokens}, {dim}]")
+            partials[i], strides[i], lds[i] = t.shape[0], n_tokens * dim, dim
+        else:
+            _rows_2d(t, "an addend")
+            if tuple(t.shape) != (n_tokens, dim):
+                raise KernelError(f"an addend {tuple(t.shape)} does not match the residual stream {tuple(h.shape)}")
+            partials[i], strides[i], lds[i] = 1, 0, (t.stride(0) if n_tokens > 1 else dim)
+        ptrs[i], dtypes[i], scales[i] = t.data_ptr(), _code(t.dtype), c
+    for name, t in (("weight", weight), ("bias", bias), ("weight2", weight2), ("bias2", bias2)):
+        if t is not None and (t.dtype != torch.float32 or t.shape != (dim,) or not t.is_contiguous()):
+            raise KernelError(f"the norm's {name} must be a contiguous float32 [{dim}] tensor")
+    if (weight is None) != (bias is None) or (weight2 is None) != (bias2 is None) or (weight is None and weight2 is not None):
+        raise KernelError("a layer norm has a weight and a bias; the second norm comes with a first")
+    if rows is not None:
+        _i32(rows, "rows")
+    n_out = n_tokens if rows is None else rows.numel()
+    out1 = torch.empty((n_out, dim), dtype=out_dtype, device=h.device) if weight is not None else None
+    out2 = torch.empty((n_out, dim), dtype=out_dtype, device=h.device) if weight2 is not None else None
+    if weight is None and not terms:
+        return None
+    lib = _build.load("layernorm")
+    _check(
+        lib,
+        lib.cwm_add_layernorm(
+            _ptr(h), ctypes.c_int(len(terms)), ptrs, dtypes, lds, partials, strides, scales, _ptr(weight), _ptr(bias), _ptr(out1),
+            _ptr(weight2), _ptr(bias2), _ptr(out2), ctypes.c_int(_code(out_dtype)), _ptr(rows), ctypes.c_int(n_out), ctypes.c_int(dim),
+            ctypes.c_float(eps), _stream(),
+        ),
+    )
+    if weight is None:
+        return None
+    return out1 if weight2 is None else (out1, out2)
+
+
+# --------------------------------------------------------------------------- #
+MAX_MEMORY_DIM = 256  # csrc/matrix_memory.hip: MEM_MAX_DIM
+
+
+def matrix_memory_state_elems(heads: int, dim: int, vdim: int) -> int:
+    """float32 values of a request's state of `heads` matrix memories of dim x vdim, in the scan kernel's own layout:
+    per head the matrix transposed, [vdim][16 * split] with split the least power of two that gives 16 * split >= dim,
+    then the normaliser's 16 * split values, then the running maximum and three unused values."""
+    split = 1
+    while 16 * split < dim:
+        split *= 2
+    return heads * (vdim * 16 * split + 16 * split + 4)
+
+
+def matrix_memory_state_unpack(flat: torch.Tensor, heads: int, dim: int, vdim: int):
+    """(S [heads, dim, vdim], n [heads, dim], m [heads]) of one request's state row (tests read states this way)."""
+    per = matrix_memory_state_elems(1, dim, vdim)
+    d_pad = (per - 4) // (vdim + 1)
+    rows = flat[: heads * per].reshape(heads, per)
+    s = rows[:, : vdim * d_pad].reshape(heads, vdim, d_pad)[:, :, :dim].transpose(1, 2)
+    return s, rows[:, vdim * d_pad : vdim * d_pad + dim], rows[:, vdim * d_pad + d_pad]
+
+
+def matrix_memory(
+    proj: torch.Tensor, gates: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, batch: Any,
+    heads: int, dim: int, vdim: int, cap: float, eps: float, q_scale: Optional[float] = None,
+) -> torch.Tensor:
+    """The matrix memory of `csrc/matrix_memory.hip` over the step's tokens.  `proj` [T, heads * (2 dim + 2 vdim)]
+    holds, side by side, queries and keys (heads * dim each), values and the output gate's projection (heads * vdim each);
+    `gates` float32 [T, 2 heads] the projections of the input gates, then of the forget gates, biases included;
+    `weight` float32 [heads * vdim]; `state` float32 [slots, >= matrix_memory_state_elems], read and written at the
+    sequences' slots.  Queries are multiplied by `q_scale` (default dim ** -0.5).  Returns [T, heads * vdim] in proj's
+    type: every head's result over its root mean square, times weight, times sigmoid(gate)."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(proj, gates, weight, state)
+    _rows_2d(proj, "the projection")
+    _rows_2d(gates, "the gates")
+    n_tokens = proj.shape[0]
+    width = heads * (2 * dim + 2 * vdim)
+    if proj.shape[1] != width or n_tokens != batch.n_tokens:
+        raise KernelError(f"the projection {tuple(proj.shape)} must be [{batch.n_tokens}, {width}]")
+    if gates.dtype != torch.float32 or tuple(gates.shape) != (n_tokens, 2 * heads):
+        raise KernelError(f"the gates must be float32 [{n_tokens}, {2 * heads}]")
+    if weight.dtype != torch.float32 or weight.shape != (heads * vdim,) or not weight.is_contiguous():
+        raise KernelError(f"the weight must be a contiguous float32 [{heads * vdim}]")
+    if dim > MAX_MEMORY_DIM:
+        raise KernelError(f"heads of {dim} rows: the scan kernel takes up to {MAX_MEMORY_DIM}")
+    need = matrix_memory_state_elems(heads, dim, vdim)
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] < need or not state.is_contiguous() or state.shape[1] % 4 != 0:
+        raise KernelError(f"the state must be a contiguous float32 [slots, >= {need}] tensor whose rows are multiples of 16 bytes")
+    coef = torch.empty((n_tokens, heads, 4), dtype=torch.float32, device=proj.device)
+    y = torch.empty((n_tokens, heads * vdim), dtype=torch.float32, device=proj.device)
+    out = torch.empty((n_tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
+    lib = _build.load("matrix_memory")
+    _check(
+        lib,
+        lib.cwm_matrix_memory(
+            _ptr(proj), ctypes.c_int(_code(proj.dtype)), ctypes.c_long(proj.stride(0) if n_tokens > 1 else width),
+            ctypes.c_int(0), ctypes.c_int(heads * dim), ctypes.c_int(2 * heads * dim), ctypes.c_int(2 * heads * dim + heads * vdim),
+            _ptr(gates), ctypes.c_long(gates.stride(0) if n_tokens > 1 else 2 * heads), ctypes.c_float(cap),
+            ctypes.c_float(dim ** -0.5 if q_scale is None else q_scale), _ptr(state), ctypes.c_long(state.shape[1]), ctypes.c_int(state.shape[0]),
+            _ptr(batch.cu_q), _ptr(batch.state_slots), ctypes.c_int(batch.n_seqs), ctypes.c_int(n_tokens),
+            _ptr(coef), _ptr(y), _ptr(weight), ctypes.c_float(eps), _ptr(out), ctypes.c_int(heads), ctypes.c_int(dim), ctypes.c_int(vdim), _stream(),
+        ),
+    )
+    return out

@@ -230,3 +230,94 @@ def qk_norm_rope_write(
         ),
     )
     return q
+
+
+def head_norm_rope_write(
+    qkv: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    qk_dim: int,
+    v_dim: int,
+    head_dim: int,
+    bias: Optional[torch.Tensor],
+    q_weight: Optional[torch.Tensor],
+    k_weight: Optional[torch.Tensor],
+    eps: float,
+    positions: torch.Tensor,
+    inv_freq: Optional[torch.Tensor],
+    out_dtype: torch.dtype,
+    cache: Optional[torch.Tensor] = None,
+    block_table: Optional[torch.Tensor] = None,
+    seq_of_token: Optional[torch.Tensor] = None,
+    v_other: Optional[torch.Tensor] = None,
+    v_mix: Optional[torch.Tensor] = None,
+    keep_values: bool = False,
+):
+    """From the joined projection `qkv` ([T, >= Hq * qk_dim + Hkv * qk_dim + Hkv * v_dim] with q, k and v leading each
+    row, or float32 partial sums [P, T, ...] of it) plus `bias` (float32, a value a column of q, k and v): every query
+    head and every key head is divided by its own root mean square (eps inside the root) and multiplied by `q_weight` /
+    `k_weight` (float32 [qk_dim], the same for all heads; None: no norm), then rotated by positions * inv_freq (float32
+    [head_dim / 2], adjacent pairs, a frequency of 0 leaves its pair alone).  With `v_other` ([T, Hkv * v_dim] of
+    `out_dtype`, rows may lie apart) and `v_mix` (one float32 on the device) the values become (1 - v_mix) v + v_mix
+    v_other.  Returns the queries [T, Hq, head_dim] in `out_dtype` (zeros from qk_dim on), and with `keep_values` also
+    the values as they were cached, [T, Hkv * v_dim]; keys and values go into the paged `cache`.  float32 arithmetic."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(qkv, bias, q_weight, k_weight, positions, inv_freq, cache, block_table, seq_of_token, v_other, v_mix)
+    width = (n_q_heads + n_kv_heads) * qk_dim + n_kv_heads * v_dim
+    n_partials, partial_stride = 1, 0
+    if qkv.dim() == 3:
+        if qkv.dtype != torch.float32 or not qkv.is_contiguous():
+            raise KernelError("partial sums must be a contiguous float32 [P, T, N] tensor")
+        n_partials, n_tokens, partial_stride, stride = qkv.shape[0], qkv.shape[1], qkv.shape[1] * qkv.shape[2], qkv.shape[2]
+    elif qkv.dim() == 2 and qkv.stride(1) == 1:
+        n_tokens, stride = qkv.shape[0], (qkv.stride(0) if qkv.shape[0] > 1 else qkv.shape[1])
+    else:
+        raise KernelError("the projection must be [T, N] with contiguous rows or partial sums [P, T, N]")
+    if qkv.shape[-1] < width:
+        raise KernelError(f"the projection has {qkv.shape[-1]} columns, the heads need {width}")
+    if head_dim % 2 != 0 or not (1 <= qk_dim <= head_dim and 1 <= v_dim <= head_dim):
+        raise KernelError(f"heads of {qk_dim} and {v_dim} do not fit an even cached head of {head_dim}")
+    _coefficients(bias, (width,), "the projections' bias")
+    _coefficients(q_weight, (qk_dim,), "the queries' norm weight")
+    _coefficients(k_weight, (qk_dim,), "the keys' norm weight")
+    _coefficients(inv_freq, (head_dim // 2,), "the rotary table")
+    _i32(positions, "positions")
+    if positions.numel() != n_tokens:
+        raise KernelError("one position per token is needed")
+    page_size = num_pages = table_width = 0
+    if cache is not None:
+        if block_table is None or seq_of_token is None:
+            raise KernelError("a cache write needs a block table and the sequence of each token")
+        if cache.dim() != 4 or cache.shape[1] != 2 or cache.shape[2] != n_kv_heads or cache.shape[3] % head_dim != 0 or not cache.is_contiguous():
+            raise KernelError(f"cache {tuple(cache.shape)} does not fit {n_kv_heads} heads of size {head_dim}")
+        if cache.dtype != out_dtype:
+            raise KernelError("the cache and the queries must have one type")
+        _i32(block_table, "block_table")
+        _i32(seq_of_token, "seq_of_token")
+        if block_table.dim() != 2 or seq_of_token.numel() != n_tokens:
+            raise KernelError("block_table must be [B, W] and seq_of_token [T]")
+        num_pages, page_size, table_width = cache.shape[0], cache.shape[3] // head_dim, block_table.shape[1]
+    if (v_other is None) != (v_mix is None):
+        raise KernelError("another layer's values and their weight come together")
+    other_stride = 0
+    if v_other is not None:
+        if v_other.dim() != 2 or tuple(v_other.shape) != (n_tokens, n_kv_heads * v_dim) or v_other.stride(1) != 1 or v_other.dtype != out_dtype:
+            raise KernelError(f"the other layer's values must be [{n_tokens}, {n_kv_heads * v_dim}] of {out_dtype}")
+        if v_mix.dtype != torch.float32 or v_mix.numel() != 1:
+            raise KernelError("the values' weight is one float32 number on the device")
+        other_stride = v_other.stride(0) if n_tokens > 1 else n_kv_heads * v_dim
+    q = torch.empty((n_tokens, n_q_heads, head_dim), dtype=out_dtype, device=qkv.device)
+    kept = torch.empty((n_tokens, n_kv_heads * v_dim), dtype=out_dtype, device=qkv.device) if keep_values else None
+    lib = _build.load("rope_kv")
+    _check(
+        lib,
+        lib.cwm_head_norm_rope_write(
+            _ptr(qkv), ctypes.c_int(_code(qkv.dtype)), ctypes.c_long(stride), ctypes.c_int(n_partials), ctypes.c_long(partial_stride),
+            _ptr(bias), _ptr(q), ctypes.c_int(_code(out_dtype)), _ptr(q_weight), _ptr(k_weight), ctypes.c_float(eps),
+            _ptr(positions), _ptr(seq_of_token), _ptr(inv_freq), _ptr(cache), _ptr(block_table),
+            ctypes.c_int(table_width), ctypes.c_int(page_size), ctypes.c_int(num_pages), ctypes.c_int(n_tokens),
+            ctypes.c_int(n_q_heads), ctypes.c_int(n_kv_heads), ctypes.c_int(qk_dim), ctypes.c_int(v_dim), ctypes.c_int(head_dim),
+            _ptr(v_other), ctypes.c_long(other_stride), _ptr(v_mix), _ptr(kept), _stream(),
+        ),
+    )
+    return (q, kept) if keep_values else q

@@ -9,6 +9,7 @@ from .base import (
     POSITION_ENCODINGS,
     Block,
     CacheSpec,
+    ChunkedKVSpec,
     Connection,
     Embedding,
     FeedForward,
@@ -30,14 +31,14 @@ from .base import (
 )
 from . import norm, rope, attention, feedforward, block, embedding, token_shift, state_space, latent_attention, experts, connection  # noqa: F401  (fill the registries)
 from .linear import LinearWeights
-from .norm import GroupRMSNorm, RMSNorm, StreamRMSNorm, StreamUpdate
+from .norm import GroupRMSNorm, LayerNorm, RMSNorm, StreamRMSNorm, StreamUpdate
 from .rope import NoPositionEncoding, RotaryEncoding, llama3_scale_frequencies, rotary_inverse_frequencies
-from .attention import PagedAttention, SinkAttention
+from .attention import HeadNormAttention, PagedAttention, SideBySide, SinkAttention
 from .feedforward import ActivatedMLP, SwiGLU
-from .block import ConnectedPreNormBlock, PostNormBlock, PreNormBlock
+from .block import ConnectedPreNormBlock, ParallelPreNormBlock, PostNormBlock, PreNormBlock
 from .connection import HyperConnection, ResidualSum
 from .embedding import LinearHead, NormedTokenEmbedding, TokenEmbedding
 from .token_shift import TokenShift
-from .state_space import SelectiveStateSpace
+from .state_space import MatrixMemory, SelectiveStateSpace
 from .latent_attention import LatentAttention
 from .experts import RoutedExperts

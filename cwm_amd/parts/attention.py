@@ -7,7 +7,7 @@ from typing import Any, Dict, Mapping, Optional
 import torch
 
 from .. import ops
-from .base import Mixer, PagedKVSpec, PartChoice, PositionEncoding, Runtime, TensorSpec, register_part
+from .base import ChunkedKVSpec, Mixer, PagedKVSpec, PartChoice, PositionEncoding, Runtime, TensorSpec, register_part
 from .linear import LinearWeights
 
 
@@ -261,3 +261,225 @@ class SinkAttention(Mixer):
 
 
 register_part("mixer", "sink_attention", SinkAttention)
+
+
+class HeadNormAttention(Mixer):
+    """Grouped-query attention over a paged cache with a norm of every query and key head, a cap on the scores, an
+    output gate, and optionally values blended with those of an earlier layer.
+
+        q = W_q x + b_q, k = W_k x + b_k, v = W_v x + b_v        `n_heads` heads of `qk_dim`, `n_kv_heads` of `qk_dim` (keys)
+                                                                 and `v_dim` (values); biases where `bias`
+        q_h <- q_h / sqrt(mean(q_h^2) + eps) * w_q, k likewise   per head, one weight of qk_dim values for all heads
+                                                                 (`qk_norm`; float32), before the rotation
+        rotation of q and k by the position encoding             its table may turn fewer than qk_dim dimensions, in
+                                                                 adjacent pairs or in halves of the turned part
+        v <- (1 - lam) v + lam v_source                          `value_mix="mix"`: v_source are the values that the layer
+                                                                 with `value_mix="source"` and the same `value_mix_key`
+                                                                 made of the same tokens in this step; lam is a stored
+                                                                 scalar; the blended v is what is cached
+        s_j = scale q . k_j;  s_j <- softcap tanh(s_j / softcap) where `softcap`
+        softmax over the keys j <= i that the mask leaves: the last `window` keys (own included), or, with `chunk`, the keys
+            of the query's own block of `chunk` positions counted from the start of the sequence; neither: all
+        out = W_o ([sum_j p_j v_j of every head] * sigmoid(W_g x))   the gate where `gate`, element by element
+
+    Keys and values are cached with one head size, the larger of qk_dim and v_dim rounded up to a multiple of 16 (zeros
+    beyond a head's own size; W_o and W_g are widened by zero columns and rows at load), so the attention kernels of
+    equal key and value heads serve it.  `names` gives the tensors' local names for the roles q, k, v, o, g, q_bias,
+    k_bias, v_bias, q_norm, k_norm and value_mix."""
+
+    replayable = True
+    DEFAULT_NAMES = {
+        "q": "q", "k": "k", "v": "v", "o": "o", "g": "g", "q_bias": "q.b", "k_bias": "k.b", "v_bias": "v.b",
+        "q_norm": "q.norm", "k_norm": "k.norm", "value_mix": "vmix",
+    }
+
+    def __init__(
+        self,
+        dim: int,
+        n_heads: int,
+        n_kv_heads: int,
+        qk_dim: int,
+        v_dim: int,
+        scale: float,
+        window: Optional[int] = None,
+        chunk: Optional[int] = None,
+        softcap: Optional[float] = None,
+        bias: bool = True,
+        qk_norm: bool = True,
+        eps: float = 1e-6,
+        gate: bool = True,
+        value_mix: Optional[str] = None,
+        value_mix_key: str = "values",
+        position_encoding: Optional[PartChoice] = None,
+        names: Optional[Mapping[str, str]] = None,
+    ) -> None:
+        if n_heads % n_kv_heads != 0:
+            raise ValueError(f"{n_heads} query heads do not divide into {n_kv_heads} key/value heads")
+        head_dim = -(-max(qk_dim, v_dim) // 16) * 16
+        if min(qk_dim, v_dim) < 1 or head_dim > MAX_HEAD_DIM:
+            raise ValueError(f"heads of {qk_dim} (queries, keys) and {v_dim} (values) are outside 1..{MAX_HEAD_DIM}, the sizes the attention kernels take")
+        if window is not None and chunk is not None:
+            raise ValueError("a window and blocks of positions exclude each other")
+        if (window is not None and window < 1) or (chunk is not None and chunk < 1):
+            raise ValueError("a window or a block holds at least the query's own key")
+        if softcap is not None and not softcap > 0:
+            raise ValueError("a cap on the scores must be positive")
+        if value_mix not in (None, "source", "mix"):
+            raise ValueError(f"value_mix {value_mix!r}: None, 'source' and 'mix' are known")
+        self.dim, self.n_heads, self.n_kv_heads = dim, n_heads, n_kv_heads
+        self.qk_dim, self.v_dim, self.head_dim = qk_dim, v_dim, head_dim
+        self.scale, self.window, self.chunk, self.softcap = float(scale), window, chunk, (float(softcap) if softcap is not None else None)
+        self.bias, self.qk_norm, self.eps, self.gate = bias, qk_norm, float(eps), gate
+        self.value_mix, self.value_mix_key = value_mix, value_mix_key
+        self.names = {**self.DEFAULT_NAMES, **dict(names or {})}
+        self.position_encoding: Optional[PositionEncoding] = (
+            position_encoding.build("position_encoding") if position_encoding is not None else None
+        )
+
+    def cache_spec(self) -> PagedKVSpec:
+        if self.chunk is not None:
+            return ChunkedKVSpec(n_kv_heads=self.n_kv_heads, head_dim=self.head_dim, chunk=self.chunk)
+        return PagedKVSpec(n_kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.window)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n = self.names
+        q_out, k_out, v_out = self.n_heads * self.qk_dim, self.n_kv_heads * self.qk_dim, self.n_kv_heads * self.v_dim
+        specs = {
+            n["q"]: TensorSpec((q_out, self.dim)),
+            n["k"]: TensorSpec((k_out, self.dim)),
+            n["v"]: TensorSpec((v_out, self.dim)),
+            n["o"]: TensorSpec((self.dim, self.n_heads * self.v_dim)),
+        }
+        if self.bias:
+            specs[n["q_bias"]] = TensorSpec((q_out,), precision="stored")
+            specs[n["k_bias"]] = TensorSpec((k_out,), precision="stored")
+            specs[n["v_bias"]] = TensorSpec((v_out,), precision="stored")
+        if self.qk_norm:
+            specs[n["q_norm"]] = TensorSpec((self.qk_dim,), init="norm", precision="stored")
+            specs[n["k_norm"]] = TensorSpec((self.qk_dim,), init="norm", precision="stored")
+        if self.gate:
+            specs[n["g"]] = TensorSpec((self.n_heads * self.v_dim, self.dim))
+        if self.value_mix is not None:  # the source layer stores the scalar too and does not use it
+            specs[n["value_mix"]] = TensorSpec((), init="zeros", precision="stored")
+        return specs
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        n = self.names
+        wq, wk, wv, wo = tensors[n["q"]], tensors[n["k"]], tensors[n["v"]], tensors[n["o"]]
+        device = wq.device
+        biases = [tensors[n[r]].float() for r in ("q_bias", "k_bias", "v_bias")] if self.bias else None
+        q_weight = tensors[n["q_norm"]].float() if self.qk_norm else None
+        k_weight = tensors[n["k_norm"]].float() if self.qk_norm else None
+        self.table: Optional[torch.Tensor] = None
+        if self.position_encoding is not None:
+            self.position_encoding.bind({}, runtime)
+            table = self.position_encoding.rotary_table()
+            if table is not None:
+                turned = 2 * table.numel()
+                if turned > self.qk_dim:
+                    raise ValueError(f"{turned} rotated dimensions exceed the head's {self.qk_dim}")
+                if self.position_encoding.rotary_pairing() == "halves":
+                    # the kernels turn adjacent elements: bring element i and i + turned / 2 of every query and key head
+                    # side by side, once, by the order of the projections' rows (and of what else is stored per element)
+                    half = turned // 2
+                    order = torch.cat([torch.stack([torch.arange(half), torch.arange(half) + half], dim=1).reshape(-1), torch.arange(turned, self.qk_dim)]).to(device)
+                    rows_q = (torch.arange(self.n_heads, device=device)[:, None] * self.qk_dim + order[None, :]).reshape(-1)
+                    rows_k = (torch.arange(self.n_kv_heads, device=device)[:, None] * self.qk_dim + order[None, :]).reshape(-1)
+                    wq, wk = wq[rows_q], wk[rows_k]
+                    if biases is not None:
+                        biases[0], biases[1] = biases[0][rows_q], biases[1][rows_k]
+                    if self.qk_norm:
+                        q_weight, k_weight = q_weight[order], k_weight[order]
+                # a frequency of 0 leaves its pair alone: the head's other dimensions, and the padding
+                self.table = torch.zeros(self.head_dim // 2, dtype=torch.float32, device=device)
+                self.table[: table.numel()] = table.to(device)
+        matrices = [wq, wk, wv]
+        if self.gate:
+            wg = tensors[n["g"]]
+            if self.v_dim != self.head_dim:  # the gate meets heads of the cached size
+                wide = torch.zeros((self.n_heads, self.head_dim, self.dim), dtype=wg.dtype, device=device)
+                wide[:, : self.v_dim] = wg.reshape(self.n_heads, self.v_dim, self.dim)
+                wg = wide.reshape(self.n_heads * self.head_dim, self.dim)
+            matrices.append(wg)
+        self.proj = LinearWeights.joined(matrices, [None] * len(matrices), stream_copy=runtime.stream_copies)
+        self.qkv_width = wq.shape[0] + wk.shape[0] + wv.shape[0]
+        self.qkv_bias = torch.cat(biases).contiguous() if biases is not None else None
+        self.q_weight = q_weight.contiguous() if q_weight is not None else None
+        self.k_weight = k_weight.contiguous() if k_weight is not None else None
+        if self.v_dim != self.head_dim:
+            wide = torch.zeros((self.dim, self.n_heads, self.head_dim), dtype=wo.dtype, device=device)
+            wide[:, :, : self.v_dim] = wo.reshape(self.dim, self.n_heads, self.v_dim)
+            wo = wide.reshape(self.dim, self.n_heads * self.head_dim)
+        self.wo = LinearWeights(wo, stream_copy=runtime.stream_copies)
+        self.lam = tensors[n["value_mix"]].float().reshape(1).contiguous() if self.value_mix == "mix" else None
+
+    def forward(self, x: torch.Tensor, batch: Any, cache: Any, write_cache: bool = True) -> torch.Tensor:
+        if not write_cache:
+            raise ValueError("this mixer writes its own cache")
+        proj = self.proj(x, partials_ok=not self.gate)
+        key = ("value_mix", self.value_mix_key)
+        v_other = None
+        if self.value_mix == "mix":
+            v_other = batch.scratch.get(key)
+            if v_other is None:
+                raise RuntimeError(f"no layer has left the values {self.value_mix_key!r} in this step")
+        result = ops.head_norm_rope_write(
+            proj, self.n_heads, self.n_kv_heads, self.qk_dim, self.v_dim, self.head_dim, self.qkv_bias, self.q_weight, self.k_weight,
+            self.eps, batch.positions, self.table, self.runtime.act_dtype, cache.cache, cache.block_table, batch.seq_of_token,
+            v_other=v_other, v_mix=self.lam, keep_values=self.value_mix == "source",
+        )
+        if self.value_mix == "source":
+            q, batch.scratch[key] = result
+        else:
+            q = result
+        attn = ops.paged_attention(q, cache.cache, cache.block_table, batch, self.window, self.scale, softcap=self.softcap, chunk=self.chunk)
+        if self.gate:
+            attn = ops.sigmoid_mul(attn, proj[:, self.qkv_width :])
+        return self.wo(attn, partials_ok=True)  # added into the residual by the next norm
+
+
+register_part("mixer", "head_norm_attention", HeadNormAttention)
+
+
+class SideBySide(Mixer):
+    """Several mixers that read the same input; the result is the sum of theirs, each times a constant:
+    sum_i scale_i mixer_i(x).  `mixers` maps a name to (the mixer chosen, its factor); a child's tensors carry its
+    name and a dot before their own.  Every child keeps a cache or state of its own (`children()` lists them in the
+    order in which `forward` takes their views); the sum is left to whoever adds the result into the residual (an
+    `ops.ScaledSum`)."""
+
+    def __init__(self, mixers: Mapping[str, Any]) -> None:
+        if not mixers:
+            raise ValueError("at least one mixer is needed")
+        self.names = list(mixers)
+        self.parts = [mixers[name][0].build("mixer") for name in self.names]
+        self.scales = [float(mixers[name][1]) for name in self.names]
+
+    @property
+    def replayable(self) -> bool:
+        return all(part.replayable for part in self.parts)
+
+    def children(self):
+        return list(self.parts)
+
+    def cache_spec(self):
+        raise TypeError("mixers side by side have a cache each; the block asks `children()`")
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {f"{name}.{t}": spec for name, part in zip(self.names, self.parts) for t, spec in part.tensor_specs().items()}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        for name, part in zip(self.names, self.parts):
+            prefix = name + "."
+            part.bind({t[len(prefix):]: v for t, v in tensors.items() if t.startswith(prefix)}, runtime)
+
+    def forward(self, x: torch.Tensor, batch: Any, cache: Any, write_cache: bool = True) -> Any:
+        views = cache if isinstance(cache, tuple) else (cache,)
+        if len(views) != len(self.parts):
+            raise ValueError(f"{len(self.parts)} mixers side by side were given {len(views)} caches")
+        return ops.ScaledSum([(part.forward(x, batch, view, write_cache), scale) for part, view, scale in zip(self.parts, views, self.scales)])
+
+
+register_part("mixer", "side_by_side", SideBySide)

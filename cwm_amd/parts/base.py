@@ -96,6 +96,28 @@ class PagedKVSpec:
 
 
 @dataclass(frozen=True)
+class ChunkedKVSpec(PagedKVSpec):
+    """Keys and values in pages for a mixer whose queries read within blocks of `chunk` positions counted from the
+    start of the sequence: the query at position p reads the keys from p - p % chunk to p, so whatever lies before
+    the block of the next token can go back to the pool."""
+
+    chunk: int = 1
+
+    def __post_init__(self) -> None:
+        if self.window is not None or self.chunk < 1:
+            raise ValueError("a cache of blocks of positions has no window, and a block holds at least one position")
+
+    def retention(self) -> Hashable:
+        return ("chunk", self.chunk)
+
+    def first_key_needed(self, length: int) -> int:
+        return length - length % self.chunk
+
+    def keys_kept(self, step_tokens: int) -> Optional[int]:
+        return self.chunk - 1 + step_tokens
+
+
+@dataclass(frozen=True)
 class StateSpec:
     """Per-request state of fixed size, zero when a request is admitted."""
 

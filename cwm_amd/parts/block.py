@@ -112,3 +112,46 @@ class ConnectedPreNormBlock(Block):
 
 
 register_part("block", "connected_pre_norm", ConnectedPreNormBlock)
+
+
+class ParallelPreNormBlock(Block):
+    """h += mixer(norm1(h)) + feed_forward(norm2(h)): both sublayers read the same residual, each through a norm of
+    its own, and their results join it in one sum.  The sum is left to the norm that reads the residual next (an
+    `ops.ScaledSum` of the sublayers' results, added in float32), and where the two norms can share their statistics
+    (`forward_pair`) one kernel makes both sublayers' inputs.  A mixer that is several side by side (it lists them
+    as `children()`) gets a cache slot for each child; a layer without a feed-forward names neither `feed_forward`
+    nor `norm2`."""
+
+    def __init__(
+        self, names: Mapping[str, str], norm1: Norm, mixer: Mixer, norm2: Optional[Norm] = None, feed_forward: Optional[FeedForward] = None,
+    ) -> None:
+        if (feed_forward is None) != (norm2 is None):
+            raise ValueError("a feed-forward and its norm come together")
+        parts = dict(norm1=norm1, mixer=mixer)
+        if feed_forward is not None:
+            parts.update(norm2=norm2, feed_forward=feed_forward)
+        super().__init__(names, **parts)
+        self.norm1, self.mixer, self.norm2, self.feed_forward = norm1, mixer, norm2, feed_forward
+
+    def mixers(self):
+        children = getattr(self.mixer, "children", None)
+        return list(children()) if children is not None else [self.mixer]
+
+    def forward(self, h: torch.Tensor, delta: Any, batch: Any, cache: Any, write_cache: bool = True) -> Any:
+        from .. import ops
+
+        if self.feed_forward is None:
+            x1, x2 = self.norm1.forward(h, delta), None
+        elif hasattr(self.norm1, "forward_pair"):
+            x1, x2 = self.norm1.forward_pair(h, delta, self.norm2)
+        else:
+            x1 = self.norm1.forward(h, delta)
+            x2 = self.norm2.forward(h, None)
+        mixed = self.mixer.forward(x1, batch, cache, write_cache)
+        terms = list(mixed.terms) if isinstance(mixed, ops.ScaledSum) else [(mixed, 1.0)]
+        if self.feed_forward is not None:
+            terms.append((self.feed_forward.forward(x2, batch), 1.0))
+        return ops.ScaledSum(terms)
+
+
+register_part("block", "parallel_pre_norm", ParallelPreNormBlock)

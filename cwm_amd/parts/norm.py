@@ -134,3 +134,42 @@ class StreamRMSNorm(RMSNorm):
 
 
 register_part("norm", "stream_rmsnorm", StreamRMSNorm)
+
+
+class LayerNorm(Norm):
+    """y = (x - mean(x)) / sqrt(var(x) + eps) * weight + bias, the variance being the mean squared deviation; float32
+    arithmetic.  The pending residual update is added first, in the same kernel and in float32; it may be a tensor,
+    partial sums, or an `ops.ScaledSum` of several sublayers' results.  `tensor` and `bias_tensor` are the local names
+    of weight and bias.  `forward_pair` serves layers whose sublayers read the same residual through norms of their
+    own: both norms share the mean and the variance, and one kernel writes both."""
+
+    replayable = True
+
+    def __init__(self, dim: int, eps: float, tensor: str = "weight", bias_tensor: str = "bias") -> None:
+        self.dim = dim
+        self.eps = float(eps)
+        self.tensor = tensor
+        self.bias_tensor = bias_tensor
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {
+            self.tensor: TensorSpec((self.dim,), init="norm", precision="stored"),
+            self.bias_tensor: TensorSpec((self.dim,), init="normal", precision="stored"),
+        }
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        self.weight = tensors[self.tensor].float().contiguous()
+        self.bias = tensors[self.bias_tensor].float().contiguous()
+
+    def forward(self, h: torch.Tensor, delta: Any, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.add_layernorm(h, delta, self.weight, self.bias, self.eps, self.runtime.act_dtype, rows)
+
+    def forward_pair(self, h: torch.Tensor, delta: Any, other: "LayerNorm"):
+        """This norm's rows and `other`'s, of the same residual after the same update."""
+        if other.dim != self.dim or other.eps != self.eps:
+            raise ValueError("two norms share their statistics only with one size and one eps")
+        return ops.add_layernorm(h, delta, self.weight, self.bias, self.eps, self.runtime.act_dtype, None, other.weight, other.bias)
+
+
+register_part("norm", "layernorm", LayerNorm)

@@ -51,13 +51,26 @@ class RotaryEncoding(PositionEncoding):
 
     replayable = True
 
-    def __init__(self, head_dim: int, theta: float, llama3_scaling: Optional[Mapping[str, float]] = None) -> None:
+    def __init__(
+        self, head_dim: int, theta: float, llama3_scaling: Optional[Mapping[str, float]] = None, linear_factor: float = 1.0,
+        pairing: str = "adjacent",
+    ) -> None:
+        """`linear_factor`: every frequency is divided by it (positions stretched by a constant).  `pairing`: which two
+        elements a frequency turns, "adjacent" (2i, 2i + 1) or "halves" (i, i + head_dim / 2); the mixer brings the
+        pairs of the second kind side by side at load, see `PositionEncoding.rotary_pairing`."""
         if head_dim % 2 != 0:
             raise ValueError("rotary pairs need an even head size")
+        if pairing not in ("adjacent", "halves"):
+            raise ValueError(f"rotary pairing {pairing!r}: 'adjacent' and 'halves' are known")
+        if not linear_factor > 0:
+            raise ValueError("the factor of a linear scaling must be positive")
         self.head_dim = head_dim
         self.theta = float(theta)
+        self.pairing = pairing
         self.llama3_scaling = dict(llama3_scaling) if llama3_scaling else None
         table = rotary_inverse_frequencies(head_dim, self.theta)
+        if linear_factor != 1.0:
+            table = table / float(linear_factor)
         if self.llama3_scaling:
             table = llama3_scale_frequencies(
                 table,
@@ -75,6 +88,9 @@ class RotaryEncoding(PositionEncoding):
 
     def rotary_table(self) -> Optional[torch.Tensor]:
         return self._table
+
+    def rotary_pairing(self) -> str:
+        return self.pairing
 
 
 class NoPositionEncoding(PositionEncoding):

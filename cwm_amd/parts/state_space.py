@@ -2,7 +2,7 @@
 
 from __future__ import annotations
 
-from typing import Any, Dict, Mapping
+from typing import Any, Dict, Mapping, Optional
 
 import torch
 
@@ -84,3 +84,68 @@ class SelectiveStateSpace(Mixer):
 
 
 register_part("mixer", "selective_state_space", SelectiveStateSpace)
+
+
+class MatrixMemory(Mixer):
+    """A matrix memory per head with exponential gates and a running maximum (the mLSTM recurrence), with a
+    per-request state.  q = W_q x * head_dim^(-1/2), k = W_k x (heads x head_dim), v = W_v x (heads x v_dim); per head
+        i_t = c tanh((W_i x + b_i) / c),   f_t = logsigmoid(c tanh((W_f x + b_f) / c))        c = `gate_cap`
+        m_t = max(f_t + m_(t-1), i_t)
+        S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T,      n_t the same with k_t alone
+        y_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)
+    with S, n and m zero at a request's start; then out = W_o (y / rms(y per head) * weight * sigmoid(W_g x)).  The
+    gates' projections leave their product in float32, and the gates, the maximum, the state, the result's norm and
+    its gate are float32 whatever the activation type.  A request's state is one float32 row in the scan kernel's own
+    layout (`ops.matrix_memory_state_elems`).  `names`: local names of the tensors for the roles q, k, v, g, o, norm,
+    i, i_bias, f, f_bias."""
+
+    replayable = True
+    DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "norm": "norm", "i": "i", "i_bias": "i.b", "f": "f", "f_bias": "f.b"}
+
+    def __init__(self, dim: int, heads: int, head_dim: int, v_dim: int, gate_cap: float, eps: float, names: Optional[Mapping[str, str]] = None) -> None:
+        if min(heads, head_dim, v_dim) < 1 or head_dim > ops.MAX_MEMORY_DIM:
+            raise ValueError(f"heads of {head_dim} x {v_dim}: the scan kernel takes 1..{ops.MAX_MEMORY_DIM} rows")
+        if not gate_cap > 0:
+            raise ValueError("the gates' cap must be positive")
+        self.dim, self.heads, self.head_dim, self.v_dim = dim, heads, head_dim, v_dim
+        self.gate_cap, self.eps = float(gate_cap), float(eps)
+        self.names = {**self.DEFAULT_NAMES, **dict(names or {})}
+        self.state_elems = ops.matrix_memory_state_elems(heads, head_dim, v_dim)
+
+    def cache_spec(self) -> StateSpec:
+        return StateSpec((self.state_elems,), torch.float32)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n = self.names
+        qk, vv = self.heads * self.head_dim, self.heads * self.v_dim
+        return {
+            n["q"]: TensorSpec((qk, self.dim)),
+            n["k"]: TensorSpec((qk, self.dim)),
+            n["v"]: TensorSpec((vv, self.dim)),
+            n["g"]: TensorSpec((vv, self.dim)),
+            n["o"]: TensorSpec((self.dim, vv)),
+            n["norm"]: TensorSpec((vv,), init="norm", precision="stored"),
+            n["i"]: TensorSpec((self.heads, self.dim)),
+            n["i_bias"]: TensorSpec((self.heads,), precision="stored"),
+            n["f"]: TensorSpec((self.heads, self.dim)),
+            n["f_bias"]: TensorSpec((self.heads,), precision="stored"),
+        }
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        n = self.names
+        self.proj = LinearWeights.joined([tensors[n[r]] for r in ("q", "k", "v", "g")], [None] * 4, stream_copy=runtime.stream_copies)
+        self.gates = LinearWeights.joined([tensors[n["i"]], tensors[n["f"]]], [tensors[n["i_bias"]], tensors[n["f_bias"]]])
+        self.w_out = LinearWeights(tensors[n["o"]], stream_copy=runtime.stream_copies)
+        self.weight = tensors[n["norm"]].float().contiguous()
+
+    def forward(self, x: torch.Tensor, batch: Any, cache: Any, write_cache: bool = True) -> torch.Tensor:
+        if not write_cache:
+            raise ValueError("a matrix memory cannot read another layer's state")
+        proj = self.proj(x)
+        gates = self.gates(x, out_dtype=torch.float32)  # float32 sums, not rounded: they enter the recurrence
+        y = ops.matrix_memory(proj, gates, self.weight, cache.state, batch, self.heads, self.head_dim, self.v_dim, self.gate_cap, self.eps)
+        return self.w_out(y, partials_ok=True)
+
+
+register_part("mixer", "matrix_memory", MatrixMemory)
