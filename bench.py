@@ -122,7 +122,9 @@ class ShapeBench:
         import torch
 
         from cwm_amd.engine import random_model
-        from cwm_amd.parts import PagedKVSpec
+        import numpy as np
+
+        from cwm_amd.parts import PagedKVSpec, StateSpec
         from cwm_amd.sampling import Sampler
 
         self.torch = torch
@@ -181,6 +183,10 @@ class ShapeBench:
                     share = next((f for prefix, f in routed.items() if name.startswith(prefix)), 1.0)
                     self.matrix_params += int(count * share)
         self.paged = [spec for spec in model.cache_specs if isinstance(spec, PagedKVSpec)]
+        # per-request state of fixed size (a recurrent mixer's): a decode step reads and writes all of it
+        self.state_bytes = sum(
+            int(np.prod(spec.shape)) * torch.empty((), dtype=spec.dtype).element_size() for spec in model.cache_specs if isinstance(spec, StateSpec)
+        )
         self.windows = sorted({spec.window for spec in self.paged if spec.window is not None})
         self.sampler = Sampler(device)
         self.vocab = model.vocab_size
@@ -195,9 +201,16 @@ class ShapeBench:
     def cache_bytes(self, batch, ctx):
         total = 0
         for spec in self.paged:
-            keys = ctx if spec.window is None else min(ctx, spec.window)
-            total += batch * keys * spec.bytes_per_token(self.esize)
-        return total
+            total += batch * self.keys_read(spec, ctx) * spec.bytes_per_token(self.esize)
+        return total + 2 * batch * self.state_bytes
+
+    @staticmethod
+    def keys_read(spec, position):
+        """Keys that the query at `position` reads of a cache with this need (its own included)."""
+        first = spec.first_key_needed(position + 1)  # what the next query could still read is what this one reads, but for
+        if spec.window is not None:                  # a window's oldest key
+            first = max(0, position - (spec.window - 1))
+        return position + 1 - first
 
     def step_bytes(self, batch, ctx):
         """What a decode step of `batch` requests at `ctx` tokens has to read: every weight once (of routed experts
@@ -214,7 +227,7 @@ class ShapeBench:
                 spec = self.model.cache_specs[slot]
                 if spec in self.paged:
                     # token p reads min(p + 1, window) keys; 2 products (QK^T and PV) of 2 flops, for every query head
-                    keys = sum(min(p + 1, spec.window or (p + 1)) for p in range(offset, offset + n_tokens))
+                    keys = sum(self.keys_read(spec, p) for p in range(offset, offset + n_tokens))
                     attn += 4 * keys * getattr(mixer, "n_heads", spec.n_kv_heads) * spec.head_dim
         return 2 * n_tokens * self.matrix_params + attn + 2 * self.head_params
 
@@ -225,8 +238,10 @@ class ShapeBench:
 
         page = self.page
         pages = {None: batch * ((ctx + extra + page - 1) // page + 1)}
-        for w in self.windows:
-            pages[w] = batch * ((min(ctx, w - 1 + step_tokens) + extra + 2 * page - 1) // page + 2)
+        for spec in self.paged:  # a group that gives pages back holds what its need keeps, and a page of slack at either end
+            kept = spec.keys_kept(step_tokens)
+            if kept is not None:
+                pages[spec.retention()] = batch * ((min(ctx, kept) + extra + 2 * page - 1) // page + 2)
         manager = CacheManager(self.model.cache_specs, page, pages, batch)
         storage = CacheStorage(manager, self.device, self.model.runtime.act_dtype)
         for t in storage.paged.values():
@@ -350,7 +365,31 @@ SEGEDRA_SIZES = {
     "w4096": (dict(width=4096, layers=8, heads=32, kv_heads=8, window=8192, streams=4, ff_dense=6144, ff=1536, experts=32, top=4), 6144),
 }
 
-COMPARISONS = {"lapevik": (LAPEVIK_SIZES, lapevik_config), "segedra": (SEGEDRA_SIZES, segedra_config)}
+def dogotar_config(width, layers, heads, kv_heads, window, block, memory_heads, ff, vocab=32768):
+    """A Dogotar model of `layers` layers in the order attention, parallel, parallel, attention: heads of 128 everywhere,
+    half of every attention head rotated, values blended across the attention layers, a dense feed-forward in every layer."""
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0, "mask": {"size": window},
+                 "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0}}, "v_mix": True}
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0, "mask": {"size": block}}
+    right = {"heads": memory_heads, "dim": 128, "vdim": 128, "gate_cap": 15.0}
+    parallel = {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}
+    mlp = {"kind": "dense", "ff": ff}
+    return {
+        "architecture": "Dogotar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+        "layers": [
+            {"type": "attention", "mixer": attention, "mlp": mlp} if i % 4 in (0, 3) else {"type": "parallel", "mixer": parallel, "mlp": mlp}
+            for i in range(layers)
+        ],
+    }
+
+
+# the same two widths; the feed-forward of two matrices is half again as wide as the dense decoder's of three, so both hold as many entries
+DOGOTAR_SIZES = {
+    "w2048": (dict(width=2048, layers=8, heads=16, kv_heads=8, window=8192, block=2048, memory_heads=16, ff=6144), 4096),
+    "w4096": (dict(width=4096, layers=8, heads=32, kv_heads=8, window=8192, block=2048, memory_heads=32, ff=9216), 6144),
+}
+
+COMPARISONS = {"lapevik": (LAPEVIK_SIZES, lapevik_config), "segedra": (SEGEDRA_SIZES, segedra_config), "dogotar": (DOGOTAR_SIZES, dogotar_config)}
 
 
 def compare_designs(args, device):
