@@ -103,7 +103,7 @@ def qkv_rope_write(x, weight, bias, n_q_heads, n_kv_heads, head_dim, positions, 
     return qkv
 
 
-def paged_attention(q, cache, block_table, batch, window, scale, sink=None):
+def paged_attention(q, cache, block_table, batch, window, scale, sink=None, softcap=None, chunk=None):
     n_tokens, n_q, hd = q.shape
     n_kv = cache.shape[2]
     page_size = cache.shape[3] // hd
@@ -113,6 +113,8 @@ def paged_attention(q, cache, block_table, batch, window, scale, sink=None):
         p = int(batch.positions[t])
         b = int(batch.seq_of_token[t])
         lo = 0 if window is None else max(0, p - (window - 1))
+        if chunk is not None:
+            lo = p - p % chunk
         keys, vals = [], []
         for j in range(lo, p + 1):
             page = int(block_table[b, j // page_size])
@@ -126,6 +128,8 @@ def paged_attention(q, cache, block_table, batch, window, scale, sink=None):
         for h in range(n_q):
             g = h // group
             s = (kk[g] @ q[t, h].float()) * scale
+            if softcap is not None:
+                s = softcap * torch.tanh(s / softcap)
             if sink is not None:  # one more term of the denominator, without a key or a value
                 w = torch.softmax(torch.cat([s, sink[h].float().reshape(1)]), -1)[:-1]
             else:
@@ -371,7 +375,100 @@ def qk_norm_rope_write(qkv, n_q_heads, n_kv_heads, qk_dim, v_dim, head_dim, q_we
     return q
 
 
+def _total(delta):
+    """A pending update (a tensor, partial sums, or a sum of scaled terms) as one float32 tensor."""
+    terms = delta.terms if hasattr(delta, "terms") else [(delta, 1.0)]
+    out = None
+    for t, c in terms:
+        x = (t.float().sum(0) if t.dim() == 3 else t.float()) * c
+        out = x if out is None else out + x
+    return out
+
+
+def add_layernorm(h, delta, weight, bias, eps, out_dtype, rows=None, weight2=None, bias2=None):
+    x = h
+    if delta is not None:
+        if rows is None:
+            h += _total(delta)
+        else:
+            x = h + _total(delta)
+    if weight is None:
+        return None
+    if rows is not None:
+        x = x[rows.long()]
+    mean = x.mean(-1, keepdim=True)
+    var = ((x - mean) ** 2).mean(-1, keepdim=True)
+    unit = (x - mean) * torch.rsqrt(var + eps)
+    first = (unit * weight.float() + bias.float()).to(out_dtype)
+    if weight2 is None:
+        return first
+    return first, (unit * weight2.float() + bias2.float()).to(out_dtype)
+
+
+def head_norm_rope_write(qkv, n_q_heads, n_kv_heads, qk_dim, v_dim, head_dim, bias, q_weight, k_weight, eps, positions, inv_freq, out_dtype,
+                         cache=None, block_table=None, seq_of_token=None, v_other=None, v_mix=None, keep_values=False):
+    if qkv.dim() == 3:
+        qkv = qkv.sum(0)
+    n = qkv.shape[0]
+    qw, kw, vw = n_q_heads * qk_dim, n_kv_heads * qk_dim, n_kv_heads * v_dim
+    qkv = qkv.float()[:, : qw + kw + vw]
+    if bias is not None:
+        qkv = qkv + bias.float()
+    q, k, v = qkv[:, :qw].reshape(n, n_q_heads, qk_dim), qkv[:, qw : qw + kw].reshape(n, n_kv_heads, qk_dim), qkv[:, qw + kw :]
+    if q_weight is not None:
+        q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * q_weight.float()
+    if k_weight is not None:
+        k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * k_weight.float()
+    if v_other is not None:
+        lam = float(v_mix.reshape(-1)[0])
+        v = (1.0 - lam) * v + lam * v_other.float()
+    kept = v.to(out_dtype)
+
+    def padded(t, heads, width):
+        out = torch.zeros((n, heads, head_dim), dtype=torch.float32)
+        out[:, :, :width] = t.reshape(n, heads, width)
+        return out
+
+    q, k, v = padded(q, n_q_heads, qk_dim), padded(k, n_kv_heads, qk_dim), padded(v, n_kv_heads, v_dim)
+    if inv_freq is not None:
+        q, k = _rotate(q, positions, inv_freq), _rotate(k, positions, inv_freq)
+    q, k, v = q.to(out_dtype), k.to(out_dtype), v.to(out_dtype)
+    if cache is not None:
+        rope_kv_write(q.clone(), k, v, positions, None, cache, block_table, seq_of_token)
+    return (q, kept) if keep_values else q
+
+
+def matrix_memory(proj, gates, weight, state, batch, heads, dim, vdim, cap, eps, q_scale=None):
+    """The state's layout is the stand-in's own: per head the matrix [dim, vdim], then the normaliser, then the maximum."""
+    n = proj.shape[0]
+    p = proj.float()
+    q = p[:, : heads * dim].reshape(n, heads, dim) * (dim ** -0.5 if q_scale is None else q_scale)
+    k = p[:, heads * dim : 2 * heads * dim].reshape(n, heads, dim)
+    v = p[:, 2 * heads * dim : 2 * heads * dim + heads * vdim].reshape(n, heads, vdim)
+    g = p[:, 2 * heads * dim + heads * vdim :].reshape(n, heads, vdim)
+    gi = cap * torch.tanh(gates.float()[:, :heads] / cap)
+    gf = torch.nn.functional.logsigmoid(cap * torch.tanh(gates.float()[:, heads:] / cap))
+    y = torch.zeros((n, heads, vdim))
+    per = dim * vdim + dim + 1
+    for b in range(batch.n_seqs):
+        row = state[int(batch.state_slots[b])]
+        for h in range(heads):
+            st = row[h * per : (h + 1) * per]
+            S, nn, m = st[: dim * vdim].reshape(dim, vdim).clone(), st[dim * vdim : dim * vdim + dim].clone(), float(st[-1])
+            for t in range(int(batch.cu_q[b]), int(batch.cu_q[b + 1])):
+                m_new = max(float(gf[t, h]) + m, float(gi[t, h]))
+                keep, take = math.exp(float(gf[t, h]) + m - m_new), math.exp(float(gi[t, h]) - m_new)
+                S = keep * S + take * torch.outer(k[t, h], v[t, h])
+                nn = keep * nn + take * k[t, h]
+                m = m_new
+                y[t, h] = (S.T @ q[t, h]) / (max(abs(float(nn @ q[t, h])), math.exp(-m)) + 1e-6)
+            st[: dim * vdim], st[dim * vdim : dim * vdim + dim], st[-1] = S.reshape(-1), nn, m
+    y = y * torch.rsqrt((y * y).mean(-1, keepdim=True) + eps)
+    return (y.reshape(n, heads * vdim) * weight.float() * torch.sigmoid(g.reshape(n, heads * vdim))).to(proj.dtype)
+
+
 STAND_INS = (
+    "add_layernorm", "head_norm_rope_write", "matrix_memory",
     "embedding_streams", "stream_mix_norm", "act_rows", "qk_norm_rope_write",
     "embedding", "add_rmsnorm", "silu_mul", "gate_up_silu", "linear", "gemm_f32", "gemm_bf16",
     "rope_kv_write", "qkv_rope_write", "paged_attention", "sample", "sample_packed", "token_logprobs",

@@ -180,17 +180,18 @@ def forward(config: dict, w: Dict[str, torch.Tensor], tokens: List[int], rounded
         p = f"l{li}."
         m = layer["mixer"]
         h1 = rd(layer_norm(x, w[p + "norm1"], w[p + "norm1.b"], eps))
-        if layer["type"] == "attention":
+        kind = layer["type"].rsplit("_", 1)[0] if layer["type"].rsplit("_", 1)[-1].isdigit() else layer["type"]  # "_<number>": other sizes
+        if kind == "attention":
             size = (m.get("mask") or {}).get("size")
             y, v_used = softmax_attention_mixer(w, p + "mix.", m, h1, eps, sliding_visible(n, size), v_first, rounded)
             if m.get("v_mix") and v_first is None:
                 v_first = v_used
-        elif layer["type"] == "parallel":
+        elif kind == "parallel":
             lm = m["left"]
             size = (lm.get("mask") or {}).get("size")
             left, _ = softmax_attention_mixer(w, p + "mix.left.", lm, h1, eps, block_visible(n, size), None, rounded)
             right = matrix_memory(w, p + "mix.right.", m["right"], h1, eps, rounded)
-            y = m["left_scale"] * left + m["right_scale"] * right
+            y = m.get("left_scale", 1.0) * left + m.get("right_scale", 1.0) * right
         else:
             raise ValueError(f"layer type {layer['type']!r}")
         if layer.get("mlp") is not None:
