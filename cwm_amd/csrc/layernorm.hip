@@ -79,10 +79,20 @@ add_layernorm_kernel(float* __restrict__ h, LnAddends addends, const float* __re
       for (int a = 0; a < addends.n; ++a) {
         const LnAddend& ad = addends.a[a];
         float y[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int p = 0; p < ad.n_partials; ++p) {
-          float z[4];
-          ln_load4(ad.ptr, ad.dtype, (size_t)p * ad.partial_stride + t * ad.ld + e, z);
-          y[0] += z[0], y[1] += z[1], y[2] += z[2], y[3] += z[3];
+        if (ad.n_partials == 1) {
+          ln_load4(ad.ptr, ad.dtype, t * ad.ld + e, y);
+        } else {
+          // four partial sums in flight at a time, added in their order; what lies beyond the last is the last again, times zero
+          for (int p = 0; p < ad.n_partials; p += 4) {
+            float z[4][4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) ln_load4(ad.ptr, ad.dtype, (size_t)min(p + u, ad.n_partials - 1) * ad.partial_stride + t * ad.ld + e, z[u]);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const float keep = p + u < ad.n_partials ? 1.0f : 0.0f;
+              y[0] = fmaf(keep, z[u][0], y[0]), y[1] = fmaf(keep, z[u][1], y[1]), y[2] = fmaf(keep, z[u][2], y[2]), y[3] = fmaf(keep, z[u][3], y[3]);
+            }
+          }
         }
         x[0] = fmaf(ad.scale, y[0], x[0]), x[1] = fmaf(ad.scale, y[1], x[1]);
         x[2] = fmaf(ad.scale, y[2], x[2]), x[3] = fmaf(ad.scale, y[3], x[3]);

@@ -8,12 +8,22 @@
 // Everything but the loads of q, k and v is float32, and tokens are walked one by one in order, so a portion of a
 // prompt gives the same bits as the same tokens one at a time.
 //
-// Two kernels.  `memory_gates_kernel` (a wavefront a (head, sequence)) walks the gates, the maximum and n, which
+// Short portions (decoding among them) are walked by two kernels.  `memory_gates_kernel` (a wavefront a (head, sequence)) walks the gates, the maximum and n, which
 // need d values a token, and leaves three numbers a token: the factor of the old state, the factor of k v^T and
 // the denominator.  `memory_scan_kernel` (a block a (tile of value columns, head, sequence)) walks S with those: a
 // thread holds 16 rows of one column, `split` lanes share a column and add their parts of S^T q by shuffles, and q,
 // k, v and the three numbers of 16 tokens are staged through LDS.  `memory_out_kernel` then divides every head's y by
 // its root mean square, multiplies by a weight and by sigmoid(gate).
+//
+// A step with a long portion takes blocks of MEMC_L tokens at once instead.  With b_t the sum of f up to t, a_s = i_s - b_s
+// and g_t = m_t - b_t, the recurrence unrolls to
+//     S_t = exp(g_c - g_t) S_c + sum_(c < s <= t) exp(a_s - g_t) k_s v_s^T        (c: the token before the block)
+// with no exponent above zero, so a block's results are (Q K^T, weighted and masked) V + (weighted Q) S_c, and the state
+// moves once a block.  `memory_maxima_kernel` walks m (a wavefront a (head, sequence), the same float32 operations as the
+// walk above, so both give the same m) and sums f in float64, since differences of long sums are taken;
+// `memory_chunk_kernel` (a block a (tile of value columns, head, sequence)) does the products in float32.  The normaliser n
+// is the column after the last value column, with ones for values, so n_t . q_t falls out as that column's result and the
+// division moves into `memory_out_kernel`.  This differs from the walk by rounding only.
 //
 // State of a request, float32: per head [e][d_pad] (S transposed: a column's rows side by side, d_pad = 16 * split),
 // then n [d_pad], then m and three unused values.
@@ -187,37 +197,221 @@ memory_scan_kernel(const T* __restrict__ src, long src_stride, int q_off, int k_
   }
 }
 
-// out[t][h * e + c] = y[t][h * e + c] / sqrt(mean_c(y[t][h]^2) + eps) * weight[h * e + c] * sigmoid(gate[t][h * e + c]);
+#define MEMC_L 32         // tokens of a block
+#define MEMC_COLS 32      // value columns of a thread block
+#define MEMC_THREADS 512
+#define MEMC_GROUPS (MEMC_THREADS / MEMC_COLS)  // groups of rows
+#define MEMC_WAVES (MEMC_THREADS / CWM_WAVE)
+
+// coef: float32 [T][heads][4]: {i_t, m_t, b_t as a float64 in two words}; b counts from the portion's start.
+// start: float64 [n_seqs][heads]: m before the portion.
+__global__ void __launch_bounds__(CWM_WAVE)
+memory_maxima_kernel(const float* __restrict__ gates, long gates_stride, float cap, float* __restrict__ state, long state_stride,
+                     long head_elems, const int* __restrict__ cu_q, const int* __restrict__ state_slots, float* __restrict__ coef,
+                     double* __restrict__ start, int heads, int e, int d_pad) {
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int t0 = cu_q[b], t1 = cu_q[b + 1];
+  float* st_m = state + (size_t)state_slots[b] * state_stride + (size_t)h * head_elems + (size_t)e * d_pad + d_pad;
+  float m = *st_m;
+  if (lane == 0) start[(size_t)b * heads + h] = (double)m;
+  const float inv_cap = 1.0f / cap;
+  double before = 0.0;
+  for (int base = t0; base < t1; base += CWM_WAVE) {
+    const int count = min(CWM_WAVE, t1 - base);
+    float gi = 0.f, gf = 0.f;
+    if (lane < count) {
+      const float* g = gates + (size_t)(base + lane) * gates_stride;
+      gi = cap * tanhf(g[h] * inv_cap);
+      gf = log_sigmoid(cap * tanhf(g[heads + h] * inv_cap));
+    }
+    double sum = (double)gf;  // zero beyond the portion's end
+#pragma unroll
+    for (int off = 1; off < CWM_WAVE; off <<= 1) {
+      const double o = __shfl_up(sum, off, CWM_WAVE);
+      if (lane >= off) sum += o;
+    }
+    float mine = 0.f;
+#pragma unroll
+    for (int j = 0; j < CWM_WAVE; ++j) {
+      if (j < count) {
+        m = fmaxf(__shfl(gf, j, CWM_WAVE) + m, __shfl(gi, j, CWM_WAVE));
+        if (lane == j) mine = m;
+      }
+    }
+    if (lane < count) {
+      float* c = coef + ((size_t)(base + lane) * heads + h) * 4;
+      c[0] = gi, c[1] = mine;
+      *(double*)(c + 2) = before + sum;
+    }
+    before += __shfl(sum, CWM_WAVE - 1, CWM_WAVE);
+  }
+  if (lane == 0) *st_m = m;
+}
+
+// y: float32 [T][heads * e], not yet divided; nq: float32 [T][heads], n_t . q_t.  RPT: rows a thread holds; 16 RPT >= d.
+template <typename T, int RPT>
+__global__ void __launch_bounds__(MEMC_THREADS)
+memory_chunk_kernel(const T* __restrict__ src, long src_stride, int q_off, int k_off, int v_off, float q_scale,
+                    const float* __restrict__ coef, const double* __restrict__ start, float* __restrict__ state, long state_stride,
+                    long head_elems, const int* __restrict__ cu_q, const int* __restrict__ state_slots, float* __restrict__ y,
+                    float* __restrict__ nq, int heads, int d, int e, int d_pad) {
+  constexpr int DP = MEMC_GROUPS * RPT, ROW = DP + 4;
+  __shared__ __attribute__((aligned(16))) float q_s[MEMC_L][ROW];
+  __shared__ __attribute__((aligned(16))) float k_s[MEMC_L][ROW];
+  __shared__ float red[MEMC_WAVES][MEMC_L][MEMC_COLS];  // (weighted Q) S_c, summed over a wavefront's two groups of rows
+  __shared__ float a_s[MEMC_L][MEMC_L + 1];             // weighted and masked scores
+  __shared__ float v_s[MEMC_L][MEMC_COLS];
+  __shared__ double ga_s[MEMC_L], gg_s[MEMC_L];         // a and g of the block's tokens
+  __shared__ float w_s[MEMC_L], dec_s[MEMC_L];          // exp(a_s - g_last), exp(g_c - g_t)
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int c = threadIdx.x & (MEMC_COLS - 1), rg = threadIdx.x / MEMC_COLS, wave = threadIdx.x / CWM_WAVE;
+  const int col = blockIdx.x * MEMC_COLS + c;  // column e is the normaliser
+  const int row0 = rg * RPT;
+  const int t0 = cu_q[b], t1 = cu_q[b + 1];
+  float* st = state + (size_t)state_slots[b] * state_stride + (size_t)h * head_elems + (size_t)col * d_pad;
+  float S[RPT];
+#pragma unroll
+  for (int j = 0; j < RPT; ++j) S[j] = (col <= e && row0 + j < d_pad) ? st[row0 + j] : 0.f;
+  double g_before = start[(size_t)b * heads + h];
+  for (int base = t0; base < t1; base += MEMC_L) {
+    const int count = min(MEMC_L, t1 - base);
+    __syncthreads();  // the block before has been read to its end
+    for (int x = threadIdx.x; x < MEMC_L * DP; x += MEMC_THREADS) {
+      const int tok = x / DP, r = x - tok * DP;
+      float qv = 0.f, kv = 0.f;
+      if (tok < count && r < d) {
+        const T* row = src + (size_t)(base + tok) * src_stride + (size_t)h * d + r;
+        qv = Elem<T>::load(row + q_off) * q_scale, kv = Elem<T>::load(row + k_off);
+      }
+      q_s[tok][r] = qv, k_s[tok][r] = kv;
+    }
+    for (int x = threadIdx.x; x < MEMC_L * MEMC_COLS; x += MEMC_THREADS) {
+      const int tok = x / MEMC_COLS, cc = blockIdx.x * MEMC_COLS + (x - tok * MEMC_COLS);
+      float vv = 0.f;
+      if (tok < count) vv = cc < e ? Elem<T>::load(src + (size_t)(base + tok) * src_stride + v_off + (size_t)h * e + cc) : (cc == e ? 1.f : 0.f);
+      v_s[tok][x - tok * MEMC_COLS] = vv;
+    }
+    if (threadIdx.x < MEMC_L) {
+      double a = -1e30, g = 1e30;  // a token beyond the end weighs nothing
+      if ((int)threadIdx.x < count) {
+        const float* cf = coef + ((size_t)(base + threadIdx.x) * heads + h) * 4;
+        const double bt = *(const double*)(cf + 2);
+        a = (double)cf[0] - bt, g = (double)cf[1] - bt;
+      }
+      ga_s[threadIdx.x] = a, gg_s[threadIdx.x] = g;
+    }
+    __syncthreads();
+    const double g_last = gg_s[count - 1];
+    {  // scores: a thread a token and two sources
+      const int t = threadIdx.x / (MEMC_L / 2), s0 = 2 * (threadIdx.x - t * (MEMC_L / 2));
+      float dot0 = 0.f, dot1 = 0.f;
+      if (s0 <= t && t < count) {
+#pragma unroll 4
+        for (int x = 0; x < DP; x += 4) {
+          const float4 qq = *(const float4*)&q_s[t][x], k0 = *(const float4*)&k_s[s0][x], k1 = *(const float4*)&k_s[s0 + 1][x];
+          dot0 = fmaf(qq.x, k0.x, dot0), dot0 = fmaf(qq.y, k0.y, dot0), dot0 = fmaf(qq.z, k0.z, dot0), dot0 = fmaf(qq.w, k0.w, dot0);
+          dot1 = fmaf(qq.x, k1.x, dot1), dot1 = fmaf(qq.y, k1.y, dot1), dot1 = fmaf(qq.z, k1.z, dot1), dot1 = fmaf(qq.w, k1.w, dot1);
+        }
+        const double g = gg_s[t];
+        dot0 *= expf((float)(ga_s[s0] - g));
+        dot1 = s0 + 1 <= t ? dot1 * expf((float)(ga_s[s0 + 1] - g)) : 0.f;
+      }
+      a_s[t][s0] = dot0, a_s[t][s0 + 1] = dot1;
+      if (threadIdx.x < MEMC_L) {
+        w_s[threadIdx.x] = expf((float)(ga_s[threadIdx.x] - g_last));
+        dec_s[threadIdx.x] = expf((float)(g_before - gg_s[threadIdx.x]));
+      }
+    }
+    __syncthreads();
+    // the old state's share of the results, then the state's own step
+    for (int t = 0; t < count; ++t) {
+      float p = 0.f;
+#pragma unroll
+      for (int j = 0; j < RPT; j += 4) {
+        const float4 qq = *(const float4*)&q_s[t][row0 + j];
+        p = fmaf(qq.x, S[j], p), p = fmaf(qq.y, S[j + 1], p), p = fmaf(qq.z, S[j + 2], p), p = fmaf(qq.w, S[j + 3], p);
+      }
+      p += __shfl_xor(p, MEMC_COLS, CWM_WAVE);
+      if ((threadIdx.x & MEMC_COLS) == 0) red[wave][t][c] = p;
+    }
+    {
+      const float keep = dec_s[count - 1];
+#pragma unroll
+      for (int j = 0; j < RPT; ++j) S[j] *= keep;
+      for (int s = 0; s < count; ++s) {
+        const float tv = w_s[s] * v_s[s][c];
+#pragma unroll
+        for (int j = 0; j < RPT; j += 4) {
+          const float4 kk = *(const float4*)&k_s[s][row0 + j];
+          S[j] = fmaf(kk.x, tv, S[j]), S[j + 1] = fmaf(kk.y, tv, S[j + 1]), S[j + 2] = fmaf(kk.z, tv, S[j + 2]), S[j + 3] = fmaf(kk.w, tv, S[j + 3]);
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < MEMC_L / MEMC_GROUPS; ++u) {
+      const int t = rg * (MEMC_L / MEMC_GROUPS) + u;
+      if (t < count && col <= e) {
+        float acc = 0.f, old = 0.f;
+        for (int s = 0; s <= t; ++s) acc = fmaf(a_s[t][s], v_s[s][c], acc);
+#pragma unroll
+        for (int w = 0; w < MEMC_WAVES; ++w) old += red[w][t][c];
+        acc = fmaf(dec_s[t], old, acc);
+        if (col < e)
+          y[(size_t)(base + t) * heads * e + (size_t)h * e + col] = acc;
+        else
+          nq[(size_t)(base + t) * heads + h] = acc;
+      }
+    }
+    g_before = g_last;
+  }
+#pragma unroll
+  for (int j = 0; j < RPT; ++j)
+    if (col <= e && row0 + j < d_pad) st[row0 + j] = S[j];
+}
+
+// out[t][h * e + c] = z[t][h * e + c] / sqrt(mean_c(z[t][h]^2) + eps) * weight[h * e + c] * sigmoid(gate[t][h * e + c]);
+// z = y, or, where nq is given (the results of `memory_chunk_kernel`), y / (max(|nq|, exp(-m)) + 1e-6) with m from coef;
 // a wavefront a (token, head)
 template <typename T>
 __global__ void __launch_bounds__(MEM_THREADS)
-memory_out_kernel(const float* __restrict__ y, const float* __restrict__ weight, const T* __restrict__ gate, long gate_stride,
-                  T* __restrict__ out, long n_pairs, int heads, int e, float eps) {
+memory_out_kernel(const float* __restrict__ y, const float* __restrict__ nq, const float* __restrict__ coef,
+                  const float* __restrict__ weight, const T* __restrict__ gate, long gate_stride, T* __restrict__ out, long n_pairs,
+                  int heads, int e, float eps) {
   const int lane = threadIdx.x & (CWM_WAVE - 1);
   const long pair = (long)blockIdx.x * (MEM_THREADS / CWM_WAVE) + threadIdx.x / CWM_WAVE;
   if (pair >= n_pairs) return;
   const long t = pair / heads;
   const int h = (int)(pair - t * heads);
   const float* row = y + (size_t)t * heads * e + (size_t)h * e;
+  const float den = nq ? fmaxf(fabsf(nq[pair]), expf(-coef[pair * 4 + 1])) + 1e-6f : 1.0f;
   float ss = 0.f;
-  for (int c = lane; c < e; c += CWM_WAVE) ss = fmaf(row[c], row[c], ss);
+  for (int c = lane; c < e; c += CWM_WAVE) {
+    const float z = nq ? row[c] / den : row[c];
+    ss = fmaf(z, z, ss);
+  }
   const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)e + eps);
   for (int c = lane; c < e; c += CWM_WAVE) {
+    const float z = nq ? row[c] / den : row[c];
     const float g = Elem<T>::load(gate + (size_t)t * gate_stride + (size_t)h * e + c);
-    Elem<T>::store(out + (size_t)t * heads * e + (size_t)h * e + c, row[c] * rstd * weight[h * e + c] / (1.0f + expf(-g)));
+    Elem<T>::store(out + (size_t)t * heads * e + (size_t)h * e + c, z * rstd * weight[h * e + c] / (1.0f + expf(-g)));
   }
 }
+
+extern "C" int cwm_matrix_memory_block_tokens() { return MEMC_L; }
 
 // src: the joined projection [n_tokens][src_stride] of dtype: q at column q_off (heads * d), k at k_off (heads * d), v at
 // v_off (heads * e), the output gate at g_off (heads * e).  gates: float32 [n_tokens][gates_stride], the input gates'
 // projection in columns 0..heads-1 and the forget gates' in heads..2 heads-1, biases included.  state: float32
 // [slots][state_stride].  coef: float32 scratch [n_tokens][heads][4]; y: float32 scratch [n_tokens][heads * e].
-// out: [n_tokens][heads * e] of dtype.
+// out: [n_tokens][heads * e] of dtype.  With `start` (float64 scratch [n_seqs][heads]) and `nq` (float32 scratch
+// [n_tokens][heads]) the portions are taken in blocks of tokens; without them they are walked token by token.
 extern "C" int cwm_matrix_memory(const void* src, int dtype, long src_stride, int q_off, int k_off, int v_off, int g_off,
                                  const float* gates, long gates_stride, float cap, float q_scale, float* state, long state_stride,
                                  int n_slots, const int* cu_q, const int* state_slots, int n_seqs, int n_tokens,
-                                 float* coef, float* y, const float* weight, float eps, void* out, int heads, int d, int e,
-                                 hipStream_t stream) {
+                                 float* coef, float* y, double* start, float* nq, const float* weight, float eps, void* out,
+                                 int heads, int d, int e, hipStream_t stream) {
   CWM_REQUIRE(heads >= 1 && d >= 1 && e >= 1 && d <= MEM_MAX_DIM, "matrix_memory: heads of %d x %d: d must lie in 1..%d", d, e, MEM_MAX_DIM);
   CWM_REQUIRE(n_seqs >= 0 && n_tokens >= 0 && n_slots >= 1, "matrix_memory: bad counts");
   CWM_REQUIRE(cap > 0.f && eps > 0.f, "matrix_memory: the gates' cap and eps must be positive");
@@ -227,22 +421,41 @@ extern "C" int cwm_matrix_memory(const void* src, int dtype, long src_stride, in
               "matrix_memory: a request's state needs %ld values, 16-byte aligned", heads * head_elems);
   CWM_REQUIRE(src && gates && state && cu_q && state_slots && coef && y && weight && out, "matrix_memory: arguments missing");
   CWM_REQUIRE(((uintptr_t)coef % 16) == 0, "matrix_memory: scratch must be 16-byte aligned");
+  CWM_REQUIRE((start == nullptr) == (nq == nullptr) && ((uintptr_t)start % 8) == 0, "matrix_memory: both scratch arrays of the blocked form, or neither");
   if (n_seqs == 0 || n_tokens == 0) return 0;
   CWM_REQUIRE(n_seqs <= 65535, "matrix_memory: too many sequences for one launch");
+  const int d_pad = MEM_ROWS * split;
   const int cols = MEM_THREADS / split;
   const int tiles = (e + cols - 1) / cols;
+  const int block_tiles = (e + 1 + MEMC_COLS - 1) / MEMC_COLS;  // the normaliser is one column more
   const long n_pairs = (long)n_tokens * heads;
   const unsigned out_blocks = (unsigned)((n_pairs + MEM_THREADS / CWM_WAVE - 1) / (MEM_THREADS / CWM_WAVE));
+#define CWM_MEMORY_BLOCKS(T, RPT)                                                                                           \
+  hipLaunchKernelGGL((memory_chunk_kernel<T, RPT>), dim3(block_tiles, heads, n_seqs), dim3(MEMC_THREADS), 0, stream,         \
+                     (const T*)src, src_stride, q_off, k_off, v_off, q_scale, (const float*)coef, (const double*)start, state, \
+                     state_stride, head_elems, cu_q, state_slots, y, nq, heads, d, e, d_pad)
 #define CWM_MEMORY(T)                                                                                                       \
   do {                                                                                                                      \
-    hipLaunchKernelGGL(memory_gates_kernel<T>, dim3(heads, n_seqs), dim3(CWM_WAVE), 0, stream, (const T*)src, src_stride,    \
-                       q_off, k_off, gates, gates_stride, cap, q_scale, state, state_stride, head_elems, cu_q, state_slots, \
-                       coef, heads, d, e, MEM_ROWS * split);                                                                \
-    hipLaunchKernelGGL(memory_scan_kernel<T>, dim3(tiles, heads, n_seqs), dim3(MEM_THREADS), 0, stream, (const T*)src,       \
-                       src_stride, q_off, k_off, v_off, q_scale, (const float*)coef, state, state_stride, head_elems, cu_q, \
-                       state_slots, y, heads, d, e, split);                                                                 \
-    hipLaunchKernelGGL(memory_out_kernel<T>, dim3(out_blocks), dim3(MEM_THREADS), 0, stream, (const float*)y, weight,        \
-                       (const T*)src + g_off, src_stride, (T*)out, n_pairs, heads, e, eps);                                 \
+    if (start) {                                                                                                            \
+      hipLaunchKernelGGL(memory_maxima_kernel, dim3(heads, n_seqs), dim3(CWM_WAVE), 0, stream, gates, gates_stride, cap,     \
+                         state, state_stride, head_elems, cu_q, state_slots, coef, start, heads, e, d_pad);                 \
+      if (d <= 4 * MEMC_GROUPS)                                                                                             \
+        CWM_MEMORY_BLOCKS(T, 4);                                                                                            \
+      else if (d <= 8 * MEMC_GROUPS)                                                                                        \
+        CWM_MEMORY_BLOCKS(T, 8);                                                                                            \
+      else                                                                                                                  \
+        CWM_MEMORY_BLOCKS(T, 16);                                                                                           \
+    } else {                                                                                                                \
+      hipLaunchKernelGGL(memory_gates_kernel<T>, dim3(heads, n_seqs), dim3(CWM_WAVE), 0, stream, (const T*)src, src_stride,  \
+                         q_off, k_off, gates, gates_stride, cap, q_scale, state, state_stride, head_elems, cu_q,            \
+                         state_slots, coef, heads, d, e, d_pad);                                                            \
+      hipLaunchKernelGGL(memory_scan_kernel<T>, dim3(tiles, heads, n_seqs), dim3(MEM_THREADS), 0, stream, (const T*)src,     \
+                         src_stride, q_off, k_off, v_off, q_scale, (const float*)coef, state, state_stride, head_elems,     \
+                         cu_q, state_slots, y, heads, d, e, split);                                                         \
+    }                                                                                                                       \
+    hipLaunchKernelGGL(memory_out_kernel<T>, dim3(out_blocks), dim3(MEM_THREADS), 0, stream, (const float*)y,                \
+                       (const float*)nq, (const float*)coef, weight, (const T*)src + g_off, src_stride, (T*)out, n_pairs,   \
+                       heads, e, eps);                                                                                      \
   } while (0)
   if (dtype == CWM_F32)
     CWM_MEMORY(float);
@@ -251,5 +464,6 @@ extern "C" int cwm_matrix_memory(const void* src, int dtype, long src_stride, in
   else
     return cwm_fail("matrix_memory: unknown type %d", dtype);
 #undef CWM_MEMORY
+#undef CWM_MEMORY_BLOCKS
   return cwm_launch_status("matrix_memory");
 }

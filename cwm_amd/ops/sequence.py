@@ -416,6 +416,7 @@ def add_layernorm(
 
 # --------------------------------------------------------------------------- #
 MAX_MEMORY_DIM = 256  # csrc/matrix_memory.hip: MEM_MAX_DIM
+MEMORY_WALK = 8  # tokens of the longest portion that a step still walks one by one; longer ones go in blocks of tokens
 
 
 def matrix_memory_state_elems(heads: int, dim: int, vdim: int) -> int:
@@ -446,7 +447,9 @@ def matrix_memory(
     `gates` float32 [T, 2 heads] the projections of the input gates, then of the forget gates, biases included;
     `weight` float32 [heads * vdim]; `state` float32 [slots, >= matrix_memory_state_elems], read and written at the
     sequences' slots.  Queries are multiplied by `q_scale` (default dim ** -0.5).  Returns [T, heads * vdim] in proj's
-    type: every head's result over its root mean square, times weight, times sigmoid(gate)."""
+    type: every head's result over its root mean square, times weight, times sigmoid(gate).  A step whose portions all
+    have up to `MEMORY_WALK` tokens (`batch.q_lens`) walks them token by token, which gives the same bits however a
+    sequence is cut; a step with a longer portion takes blocks of tokens at once, which differs from the walk by rounding."""
     KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
     _need_gpu(proj, gates, weight, state)
     _rows_2d(proj, "the projection")
@@ -467,6 +470,11 @@ def matrix_memory(
     coef = torch.empty((n_tokens, heads, 4), dtype=torch.float32, device=proj.device)
     y = torch.empty((n_tokens, heads * vdim), dtype=torch.float32, device=proj.device)
     out = torch.empty((n_tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
+    start = nq = None
+    q_lens = getattr(batch, "q_lens", None)
+    if q_lens and max(q_lens) > MEMORY_WALK:
+        start = torch.empty((batch.n_seqs, heads), dtype=torch.float64, device=proj.device)
+        nq = torch.empty((n_tokens, heads), dtype=torch.float32, device=proj.device)
     lib = _build.load("matrix_memory")
     _check(
         lib,
@@ -476,7 +484,8 @@ def matrix_memory(
             _ptr(gates), ctypes.c_long(gates.stride(0) if n_tokens > 1 else 2 * heads), ctypes.c_float(cap),
             ctypes.c_float(dim ** -0.5 if q_scale is None else q_scale), _ptr(state), ctypes.c_long(state.shape[1]), ctypes.c_int(state.shape[0]),
             _ptr(batch.cu_q), _ptr(batch.state_slots), ctypes.c_int(batch.n_seqs), ctypes.c_int(n_tokens),
-            _ptr(coef), _ptr(y), _ptr(weight), ctypes.c_float(eps), _ptr(out), ctypes.c_int(heads), ctypes.c_int(dim), ctypes.c_int(vdim), _stream(),
+            _ptr(coef), _ptr(y), _ptr(start), _ptr(nq), _ptr(weight), ctypes.c_float(eps), _ptr(out), ctypes.c_int(heads), ctypes.c_int(dim),
+            ctypes.c_int(vdim), _stream(),
         ),
     )
     return out

@@ -127,23 +127,15 @@ def softmax_attention_mixer(
     return rd(mixed @ w[p + "o"].T), v
 
 
-def matrix_memory(
-    w: Dict[str, torch.Tensor], p: str, m: dict, h: torch.Tensor, eps: float, rounded: bool = False
-) -> torch.Tensor:
-    """Per head, with S [d, e], n [d] and a running maximum r, all zero before the first token:
-        i_t = c tanh((W_i h + b_i) / c),  f_t = logsigmoid(c tanh((W_f h + b_f) / c))
+def memory_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gi: torch.Tensor, gf: torch.Tensor) -> torch.Tensor:
+    """q (already scaled), k [T, H, d], v [T, H, e], log input and forget gates gi, gf [T, H].  Per head, with S [d, e],
+    n [d] and a running maximum r, all zero before the first token:
         r_t = max(f_t + r_(t-1), i_t)
         S_t = exp(f_t + r_(t-1) - r_t) S_(t-1) + exp(i_t - r_t) k_t v_t^T,   n_t likewise with k_t
-        o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-r_t)) + 1e-6),   q = W_q h / sqrt(d)
-    then every head's o over its root mean square, all heads times the weight, times sigmoid(W_g h), then W_o."""
-    T = h.shape[0]
-    H, d, e, c = m["heads"], m["dim"], m["vdim"], m["gate_cap"]
-    rd = bf16_round if rounded else (lambda t: t)
-    q = rd(h @ w[p + "q"].T).reshape(T, H, d) * d ** -0.5
-    k = rd(h @ w[p + "k"].T).reshape(T, H, d)
-    v = rd(h @ w[p + "v"].T).reshape(T, H, e)
-    gi = c * torch.tanh((h @ w[p + "i"].T + w[p + "i.b"]) / c)
-    gf = torch.nn.functional.logsigmoid(c * torch.tanh((h @ w[p + "f"].T + w[p + "f.b"]) / c))
+        o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-r_t)) + 1e-6)
+    Returns o [T, H, e]."""
+    T, H, d = k.shape
+    e = v.shape[2]
     out = torch.zeros(T, H, e, dtype=F)
     for a in range(H):
         S = torch.zeros(d, e, dtype=F)
@@ -158,6 +150,29 @@ def matrix_memory(
             r = r_new
             den = max(abs(float(nrm @ q[t, a])), math.exp(-r)) + 1e-6
             out[t, a] = (S.T @ q[t, a]) / den
+    return out
+
+
+def capped_log_gates(w: Dict[str, torch.Tensor], p: str, h: torch.Tensor, c: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """i = c tanh((W_i h + b_i) / c),  f = logsigmoid(c tanh((W_f h + b_f) / c)), [T, H] each."""
+    gi = c * torch.tanh((h @ w[p + "i"].T + w[p + "i.b"]) / c)
+    gf = torch.nn.functional.logsigmoid(c * torch.tanh((h @ w[p + "f"].T + w[p + "f.b"]) / c))
+    return gi, gf
+
+
+def matrix_memory(
+    w: Dict[str, torch.Tensor], p: str, m: dict, h: torch.Tensor, eps: float, rounded: bool = False
+) -> torch.Tensor:
+    """q = W_q h / sqrt(d), k = W_k h, v = W_v h and capped log gates enter `memory_recurrence`; then every head's o
+    over its root mean square, all heads times the weight, times sigmoid(W_g h), then W_o."""
+    T = h.shape[0]
+    H, d, e, c = m["heads"], m["dim"], m["vdim"], m["gate_cap"]
+    rd = bf16_round if rounded else (lambda t: t)
+    q = rd(h @ w[p + "q"].T).reshape(T, H, d) * d ** -0.5
+    k = rd(h @ w[p + "k"].T).reshape(T, H, d)
+    v = rd(h @ w[p + "v"].T).reshape(T, H, e)
+    gi, gf = capped_log_gates(w, p, h, c)
+    out = memory_recurrence(q, k, v, gi, gf)
     y = unit_rms(out, eps).reshape(T, H * e) * w[p + "norm"]
     y = rd(y * torch.sigmoid(rd(h @ w[p + "g"].T)))
     return rd(y @ w[p + "o"].T)
