@@ -419,6 +419,16 @@ MAX_MEMORY_DIM = 256  # csrc/matrix_memory.hip: MEM_MAX_DIM
 MEMORY_WALK = 8  # tokens of the longest portion that a step still walks one by one; longer ones go in blocks of tokens
 
 
+_MEMORY_BLOCK_TOKENS = None
+
+
+def _memory_block_tokens() -> int:
+    global _MEMORY_BLOCK_TOKENS
+    if _MEMORY_BLOCK_TOKENS is None:
+        _MEMORY_BLOCK_TOKENS = int(_build.load("matrix_memory").cwm_matrix_memory_block_tokens())
+    return _MEMORY_BLOCK_TOKENS
+
+
 def matrix_memory_state_elems(heads: int, dim: int, vdim: int) -> int:
     """float32 values of a request's state of `heads` matrix memories of dim x vdim, in the scan kernel's own layout:
     per head the matrix transposed, [vdim][16 * split] with split the least power of two that gives 16 * split >= dim,
@@ -470,11 +480,12 @@ def matrix_memory(
     coef = torch.empty((n_tokens, heads, 4), dtype=torch.float32, device=proj.device)
     y = torch.empty((n_tokens, heads * vdim), dtype=torch.float32, device=proj.device)
     out = torch.empty((n_tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
-    start = nq = None
+    start = nq = scores = None
     q_lens = getattr(batch, "q_lens", None)
     if q_lens and max(q_lens) > MEMORY_WALK:
         start = torch.empty((batch.n_seqs, heads), dtype=torch.float64, device=proj.device)
         nq = torch.empty((n_tokens, heads), dtype=torch.float32, device=proj.device)
+        scores = torch.empty((n_tokens, heads, _memory_block_tokens() + 2), dtype=torch.float32, device=proj.device)
     lib = _build.load("matrix_memory")
     _check(
         lib,
@@ -484,7 +495,7 @@ def matrix_memory(
             _ptr(gates), ctypes.c_long(gates.stride(0) if n_tokens > 1 else 2 * heads), ctypes.c_float(cap),
             ctypes.c_float(dim ** -0.5 if q_scale is None else q_scale), _ptr(state), ctypes.c_long(state.shape[1]), ctypes.c_int(state.shape[0]),
             _ptr(batch.cu_q), _ptr(batch.state_slots), ctypes.c_int(batch.n_seqs), ctypes.c_int(n_tokens),
-            _ptr(coef), _ptr(y), _ptr(start), _ptr(nq), _ptr(weight), ctypes.c_float(eps), _ptr(out), ctypes.c_int(heads), ctypes.c_int(dim),
+            _ptr(coef), _ptr(y), _ptr(start), _ptr(nq), _ptr(scores), _ptr(weight), ctypes.c_float(eps), _ptr(out), ctypes.c_int(heads), ctypes.c_int(dim),
             ctypes.c_int(vdim), _stream(),
         ),
     )
