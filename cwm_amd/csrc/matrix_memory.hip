@@ -345,6 +345,13 @@ memory_scores_kernel(const T* __restrict__ src, long src_stride, int q_off, int 
 
 typedef float memc_acc __attribute__((ext_vector_type(16)));
 
+__device__ __forceinline__ float raw_to_f32(float x) { return x; }
+__device__ __forceinline__ float raw_to_f32(bf16_t x) { return bf16_to_f32(x); }
+
+// A barrier that waits for the wavefront's LDS accesses only: __syncthreads() also waits for every global load on its
+// way, which here are the next block's rows, fetched early so that they arrive during this block's products.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory"); }
+
 // y: float32 [T][heads * e], not yet divided; nq: float32 [T][heads], n_t . q_t.  TILES wavefronts a thread block, each with
 // 32 rows of the block's 32 columns of S in the registers of a 32 x 32 float32 matrix instruction's result (lane l, register r:
 // row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32); 32 TILES >= d.  A block of tokens takes three chains of such
@@ -380,51 +387,51 @@ memory_chunk_kernel(const T* __restrict__ src, long src_stride, int q_off, int k
     const int row = tile_row + 8 * (r / 4) + 4 * half + (r % 4);
     S[r] = (col <= e && row < d_pad) ? st[row] : 0.f;
   }
-  float q_r[QK_REGS], k_r[QK_REGS], v_r[V_REGS], a_r[V_REGS], w_r = 0.f, dec_r = 0.f;
+  // What a fetch leaves in registers is what the loads return and nothing made of it: an operation on a loaded value would
+  // wait for the load where the fetch is issued, not where the value is staged.  Every load is issued, from an address that
+  // exists; conversion, scale and the zeros beyond the portion's end or the head's size are applied when the block is staged.
+  T q_r[QK_REGS], k_r[QK_REGS], v_r[V_REGS];
+  float a_r[V_REGS];
+  float2 wd_r = make_float2(0.f, 0.f);
   auto fetch = [&](int base) {
     const int count = min(MEMC_L, t1 - base);
 #pragma unroll
     for (int u = 0; u < QK_REGS; ++u) {
       const int x = threadIdx.x + u * THREADS, tok = x / DP, r = x - tok * DP;
-      // every load is issued, from an address that exists, and what it should not have read is dropped afterwards:
-      // loads under conditions would wait for one another
-      const bool live = tok < count && r < d;
       const T* row = src + (size_t)(base + min(tok, count - 1)) * src_stride + (size_t)h * d + min(r, d - 1);
-      const float qv = Elem<T>::load(row + q_off), kv = Elem<T>::load(row + k_off);
-      q_r[u] = live ? qv * q_scale : 0.f, k_r[u] = live ? kv : 0.f;
+      q_r[u] = row[q_off], k_r[u] = row[k_off];
     }
 #pragma unroll
     for (int u = 0; u < V_REGS; ++u) {
       const int x = threadIdx.x + u * THREADS, tok = x / MEMC_COLS, cc = blockIdx.x * MEMC_COLS + (x - tok * MEMC_COLS);
       const size_t at = (size_t)(base + min(tok, count - 1));
-      const float vv = Elem<T>::load(src + at * src_stride + v_off + (size_t)h * e + min(cc, e - 1));
-      const float aa = scores[(at * heads + h) * MEMC_L + (x - tok * MEMC_COLS)];
-      v_r[u] = tok < count ? (cc < e ? vv : (cc == e ? 1.f : 0.f)) : 0.f;
-      a_r[u] = tok < count ? aa : 0.f;
+      v_r[u] = src[at * src_stride + v_off + (size_t)h * e + min(cc, e - 1)];
+      a_r[u] = scores[(at * heads + h) * MEMC_L + (x - tok * MEMC_COLS)];
     }
-    {
-      const float2 p = *(const float2*)(wd + ((size_t)(base + min((int)threadIdx.x, count - 1)) * heads + h) * 2);
-      const bool live = (int)threadIdx.x < count;
-      w_r = live ? p.x : 0.f, dec_r = live ? p.y : 0.f;
-    }
+    wd_r = *(const float2*)(wd + ((size_t)(base + min((int)threadIdx.x, count - 1)) * heads + h) * 2);
   };
   if (t0 < t1) fetch(t0);
   for (int base = t0; base < t1; base += MEMC_L) {
     const int count = min(MEMC_L, t1 - base);
-    __syncthreads();  // the block before has been read to its end
+    lds_barrier();  // the block before has been read to its end
 #pragma unroll
     for (int u = 0; u < QK_REGS; ++u) {
       const int x = threadIdx.x + u * THREADS, tok = x / DP, r = x - tok * DP;
-      q_s[tok][r] = q_r[u], k_s[tok][r] = k_r[u];
+      const bool live = tok < count && r < d;
+      q_s[tok][r] = live ? raw_to_f32(q_r[u]) * q_scale : 0.f, k_s[tok][r] = live ? raw_to_f32(k_r[u]) : 0.f;
     }
 #pragma unroll
     for (int u = 0; u < V_REGS; ++u) {
-      const int x = threadIdx.x + u * THREADS, tok = x / MEMC_COLS;
-      v_s[tok][x - tok * MEMC_COLS] = v_r[u], a_s[tok][x - tok * MEMC_COLS] = a_r[u];
+      const int x = threadIdx.x + u * THREADS, tok = x / MEMC_COLS, cl = x - tok * MEMC_COLS, cc = blockIdx.x * MEMC_COLS + cl;
+      v_s[tok][cl] = tok < count ? (cc < e ? raw_to_f32(v_r[u]) : (cc == e ? 1.f : 0.f)) : 0.f;
+      a_s[tok][cl] = tok < count ? a_r[u] : 0.f;
     }
-    if (threadIdx.x < MEMC_L) w_s[threadIdx.x] = w_r, dec_s[threadIdx.x] = dec_r;
+    if (threadIdx.x < MEMC_L) {
+      const bool live = (int)threadIdx.x < count;
+      w_s[threadIdx.x] = live ? wd_r.x : 0.f, dec_s[threadIdx.x] = live ? wd_r.y : 0.f;
+    }
     if (base + MEMC_L < t1) fetch(base + MEMC_L);  // on its way during this block's products
-    __syncthreads();
+    lds_barrier();
     // what lies beyond the portion's end was staged as zeros, so every chain runs over the whole block
     memc_acc part;
 #pragma unroll
@@ -455,7 +462,8 @@ memory_chunk_kernel(const T* __restrict__ src, long src_stride, int q_off, int k
         S = __builtin_amdgcn_mfma_f32_32x32x2f32(k_s[s][tile_row + c], w_s[s] * v_s[s][c], S, 0, 0, 0);
       }
     }
-    __syncthreads();
+    lds_barrier();
+
     for (int x = threadIdx.x; x < MEMC_L * MEMC_COLS; x += THREADS) {
       const int t = x / MEMC_COLS, cc = x - t * MEMC_COLS, out_col = blockIdx.x * MEMC_COLS + cc;
       if (t < count && out_col <= e) {
