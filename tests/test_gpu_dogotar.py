@@ -366,6 +366,20 @@ def test_a_loud_key_at_a_window_s_edges_under_the_cap(window, page_size):
         _both_attention_kernels(dtype, hd, page_size, case, window, None, 25.0, f"window {window}")
 
 
+@pytest.mark.parametrize("block", [None, 8192])
+def test_a_loud_key_far_back_under_the_cap_where_key_ranges_are_cut_and_merged(block):
+    """Decoded tokens and portions far into long sequences: the matrix-core kernel cuts their keys into ranges and a
+    second kernel merges the partial results, the plain kernel cuts into segments.  One key thousands of places back
+    (with blocks: at the first place of the query's block) carries the last row of a decoded token and of a portion."""
+    n_q, n_kv, hd, page_size = 6, 2, 64, 64
+    lens_old, lens_new = [9000, 3000, 1500, 20000, 9000], [1, 2, 1, 150, 600]
+    loud = [(0, 8192 if block else 4321), (4, 8192 if block else 77)]
+    case = _attention_case(torch.bfloat16, n_q, n_kv, hd, page_size, lens_old, lens_new, None, block, 25.0, seed=5, loud=loud)
+    quiet = _attention_case(torch.bfloat16, n_q, n_kv, hd, page_size, lens_old, lens_new, None, block, 25.0, seed=5)[-1]
+    assert (quiet[0] - case[-1][0]).abs().max() > 0.3 and (quiet[-1] - case[-1][-1]).abs().max() > 0.3
+    _both_attention_kernels(torch.bfloat16, hd, page_size, case, None, block, 25.0, f"far key, block {block}")
+
+
 # ---- models ------------------------------------------------------------------------------------------------------- #
 LENGTHS = {"tiny_d": [1, 6, 21, 70, 130], "tiny_e": [9, 33, 2, 100, 57], "tiny_f": [150, 41, 90]}
 PAGE_SIZES = {"whole": 16, "tail": 16, "portions": 8, "mixed": 8}
