@@ -471,7 +471,7 @@ extern "C" int cwm_qk_norm_rope_write(const void* src, int src_dtype, long src_s
               "qk_norm_rope_write: head_dim %d must be even and at most %d", head_dim, NORM_ROPE_MAX_HEAD);
   CWM_REQUIRE(qk_dim >= 1 && v_dim >= 1 && qk_dim <= head_dim && v_dim <= head_dim,
               "qk_norm_rope_write: heads of %d (queries, keys) and %d (values) do not fit the cached head of %d", qk_dim, v_dim, head_dim);
-  CWM_REQUIRE(n_q_heads > 0 && n_kv_heads > 0, "qk_norm_rope_write: no heads");
+  CWM_REQUIRE(n_q_heads > 0 && (n_kv_heads > 0 || (n_kv_heads == 0 && !cache)), "qk_norm_rope_write: no heads");
   CWM_REQUIRE(src && q_out && positions, "qk_norm_rope_write: arguments missing");
   CWM_REQUIRE(eps > 0.f || (!q_weight && !k_weight), "qk_norm_rope_write: eps must be positive");
   if (cache) {

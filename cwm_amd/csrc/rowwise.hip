@@ -424,3 +424,66 @@ extern "C" int cwm_act_rows(void* out, int out_dtype, const void* x, int x_dtype
 #undef CWM_ACT_LAUNCH
   return cwm_launch_status("act_rows");
 }
+
+// ---- out = gated(sum over p of x[p]) ------------------------------------------------ //
+// What a gated feed-forward makes of its joined gate/up product: `x` is [T, 2 F (+ extra)] of type TX, a row's gate
+// values first, then its up values (or n_partials float32 slabs that are added in order first); out [T, F].
+// kind 0: silu(g) * u.  kind 1: g' * sigmoid(alpha * g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit,
+// limit).  With `row_gate_col` >= 0 the row is also multiplied by the sigmoid of that column of x (one more output
+// of the same product: a gate on the whole row).  float32 arithmetic, rounded once.
+__device__ __forceinline__ float gated_pair(float g, float u, int kind, float alpha, float limit) {
+  if (kind == 1) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + expf(-alpha * g)) * (u + 1.f);
+  }
+  return g / (1.f + expf(-g)) * u;
+}
+
+template <typename TX, typename TO>
+__global__ void gated_act_rows_kernel(TO* __restrict__ out, const TX* __restrict__ x, long x_ld, int n_partials,
+                                      long partial_stride, int n_rows, int hidden, int row_gate_col, int kind, float alpha,
+                                      float limit) {
+  const long count = (long)n_rows * hidden;
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (; i < count; i += stride) {
+    const long t = i / hidden;
+    const int f = (int)(i - t * hidden);
+    const TX* row = x + (size_t)t * x_ld;
+    float g = 0.f, u = 0.f, r = 0.f;
+    for (int p = 0; p < n_partials; ++p) {
+      g += Elem<TX>::load(row + (size_t)p * partial_stride + f);
+      u += Elem<TX>::load(row + (size_t)p * partial_stride + hidden + f);
+      if (row_gate_col >= 0) r += Elem<TX>::load(row + (size_t)p * partial_stride + row_gate_col);
+    }
+    float v = gated_pair(g, u, kind, alpha, limit);
+    if (row_gate_col >= 0) v *= 1.f / (1.f + expf(-r));
+    Elem<TO>::store(out + i, v);
+  }
+}
+
+extern "C" int cwm_gated_act_rows(void* out, int out_dtype, const void* x, int x_dtype, long x_ld, int n_partials,
+                                  long partial_stride, int n_rows, int hidden, int row_gate_col, int kind, float alpha,
+                                  float limit, hipStream_t stream) {
+  CWM_REQUIRE(n_partials >= 1 && n_rows >= 0 && hidden >= 1, "gated_act_rows: bad sizes");
+  CWM_REQUIRE(n_partials == 1 || x_dtype == CWM_F32, "gated_act_rows: partial sums must be float32");
+  CWM_REQUIRE(kind == 0 || kind == 1, "gated_act_rows: unknown gated activation %d", kind);
+  CWM_REQUIRE(kind == 0 || limit > 0.f, "gated_act_rows: the clamped form needs a positive limit");
+  if (n_rows == 0) return 0;
+  long blocks = ((long)n_rows * hidden + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  const int key = (x_dtype << 1) | out_dtype;
+#define CWM_GACT_LAUNCH(TX, TO)                                                                                         \
+  hipLaunchKernelGGL((gated_act_rows_kernel<TX, TO>), dim3((unsigned)blocks), dim3(256), 0, stream, (TO*)out, (const TX*)x, \
+                     x_ld, n_partials, partial_stride, n_rows, hidden, row_gate_col, kind, alpha, limit)
+  switch (key) {
+    case 0: CWM_GACT_LAUNCH(float, float); break;
+    case 1: CWM_GACT_LAUNCH(float, bf16_t); break;
+    case 2: CWM_GACT_LAUNCH(bf16_t, float); break;
+    case 3: CWM_GACT_LAUNCH(bf16_t, bf16_t); break;
+    default: return cwm_fail("gated_act_rows: unknown dtypes x=%d out=%d", x_dtype, out_dtype);
+  }
+#undef CWM_GACT_LAUNCH
+  return cwm_launch_status("gated_act_rows");
+}

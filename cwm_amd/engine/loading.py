@@ -51,7 +51,7 @@ def wants_stream_copies(model: Model, act_dtype: torch.dtype, device: torch.devi
     matrix_bytes = 0
     for spec in model.tensor_specs().values():
         if len(spec.shape) == 2 and spec.kind == "float":
-            matrix_bytes += 2 * spec.shape[0] * spec.shape[1]
+            matrix_bytes += 2 * abs(spec.shape[0] * spec.shape[1])
     total = torch.cuda.get_device_properties(device).total_memory
     return 2 * matrix_bytes <= STREAM_COPY_SHARE * total
 

@@ -1,4 +1,4 @@
 from .model import Model
-from . import llama3_dense, lapevik, segedra, dogotar  # noqa: F401  (register the architectures)
+from . import llama3_dense, lapevik, segedra, dogotar, digasun  # noqa: F401  (register the architectures)
 
 __all__ = ["Model"]

@@ -7,7 +7,7 @@ from typing import Dict, List, Mapping, Optional, Set, Tuple
 
 import torch
 
-from ..parts.base import BLOCKS, Block, CacheSpec, Embedding, Head, LayerCall, ModelPlan, Norm, Part, Runtime, TensorSpec
+from ..parts.base import BLOCKS, Block, CacheSpec, Embedding, Head, LayerCall, ModelPlan, Norm, Part, Runtime, TensorSpec, is_absolute
 
 
 class Model:
@@ -34,7 +34,7 @@ class Model:
         # run order: entry i runs block `layer` on the cache slots `cache_slots[i]`, one for each of the block's mixers
         self.run_order: List[LayerCall] = list(plan.run_order)
         self.cache_slots: List[Tuple[int, ...]] = []
-        self.writes_cache: List[bool] = []
+        self.writes_cache: List[object] = []  # a boolean an entry, or one a mixer where only some read another entry's cache
         self.cache_specs: List[CacheSpec] = []
         owner_slots: Dict[int, Tuple[int, ...]] = {}
         for i, call in enumerate(self.run_order):
@@ -42,10 +42,34 @@ class Model:
                 raise ValueError(f"run order entry {i} names layer {call.layer}, the model has {len(self.blocks)}")
             specs = [mixer.cache_spec() for mixer in self.blocks[call.layer].mixers()]
             if call.cache_of is None:
+                if call.shared_mixers is not None:
+                    raise ValueError(f"run order entry {i} names shared mixers and no entry whose cache they read")
                 owner_slots[i] = tuple(range(len(self.cache_specs), len(self.cache_specs) + len(specs)))
                 self.cache_specs.extend(specs)
                 self.cache_slots.append(owner_slots[i])
                 self.writes_cache.append(True)
+            elif call.shared_mixers is not None:
+                if call.cache_of not in owner_slots:
+                    raise ValueError(
+                        f"run order entry {i} reads the cache of entry {call.cache_of}, "
+                        "which is not an earlier entry with a cache of its own"
+                    )
+                theirs = owner_slots[call.cache_of]
+                slots, writes = [], []
+                for m, spec in enumerate(specs):
+                    if m in call.shared_mixers:
+                        if m >= len(theirs) or self.cache_specs[theirs[m]] != spec:
+                            raise ValueError(f"run order entry {i}: mixer {m} cannot read a cache of another shape (entry {call.cache_of})")
+                        slots.append(theirs[m])
+                        writes.append(False)
+                    else:
+                        slots.append(len(self.cache_specs))
+                        self.cache_specs.append(spec)
+                        writes.append(True)
+                if any(not 0 <= m < len(specs) for m in call.shared_mixers):
+                    raise ValueError(f"run order entry {i} shares mixers {call.shared_mixers}, its block has {len(specs)}")
+                self.cache_slots.append(tuple(slots))
+                self.writes_cache.append(tuple(writes))
             else:
                 if call.cache_of not in owner_slots:
                     raise ValueError(
@@ -83,7 +107,7 @@ class Model:
                 add(prefix + name, spec)
         for layer, block in zip(self.plan.layers, self.blocks):
             for name, spec in block.tensor_specs().items():
-                add(layer.prefix + name, spec)
+                add(name[1:] if is_absolute(name) else layer.prefix + name, spec)
         for name, spec in self.final_norm.tensor_specs().items():
             add(self.plan.final_norm.prefix + name, spec)
         return specs
@@ -99,7 +123,9 @@ class Model:
         self.runtime = runtime
         for layer, block in zip(self.plan.layers, self.blocks):
             prefix = layer.prefix
-            block.bind({n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}, runtime)
+            own = {n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}
+            own.update({n: tensors[n[1:]] for n in block.tensor_specs() if is_absolute(n)})
+            block.bind(own, runtime)
         for _role, prefix, part in self._ends:
             names = part.tensor_specs()
             part.bind({name: tensors[prefix + name] for name in names}, runtime)

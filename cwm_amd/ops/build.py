@@ -61,6 +61,10 @@ SOURCES: Dict[str, Tuple[Mapping[str, int], ...]] = {
     "streams": ({},),
     "layernorm": ({},),
     "matrix_memory": ({},),
+    "attention_talk": ({},),
+    "linear_attention": ({},),
+    "short_conv": ({},),
+    "token_side": ({},),
     "attention_mfma": tuple({"HEAD_DIM": hd} for hd in (16, 32, 48, 64, 80, 96, 128, 256)),
 }
 

@@ -1,0 +1,272 @@
+"""Entry points of the kernels of layers whose attention heads exchange their weights, of gated linear attention, of
+short input convolutions, of a layer's own token input and of gated activations on rows
+(`csrc/attention_talk.hip`, `csrc/linear_attention.hip`, `csrc/short_conv.hip`, `csrc/token_side.hip`, `csrc/rowwise.hip`).
+Shapes, types and devices are checked on the host; there is no CPU path."""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Any, Optional, Sequence, Tuple
+
+import torch
+
+from . import build as _build
+
+MAX_TALK_HEADS = 64  # csrc/attention_talk.hip: TALK_MAX_HEADS
+TALK_SPLIT = 128  # csrc/attention_talk.hip: keys of a range of a token's keys
+MAX_SHORT_CONV_TAPS = 16  # csrc/short_conv.hip: SCONV_MAX_TAPS
+MAX_GLA_DIM = 256  # csrc/linear_attention.hip: GLA_MAX_DIM
+MAX_SIDE_DIM = 256  # csrc/token_side.hip: SIDE_MAX_DIM
+
+
+def _base():
+    from . import KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream  # the shared helpers of this package
+
+    return KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream
+
+
+def talking_attention(
+    q: torch.Tensor,
+    cache: torch.Tensor,
+    block_table: torch.Tensor,
+    batch: Any,
+    window: Optional[int],
+    scale: float,
+    sink: Optional[torch.Tensor] = None,
+    talk: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Causal attention of `q` [T, Hq, hd] over the paged cache ([pages, 2, Hkv, page * hd]) whose heads mix their
+    softmax weights: head h applies sum_g talk[h, g] p_g to the values of its own key/value head, with
+    p_g = exp(scale q_g . k) / (sum over the `window` keys up to the query's own + exp(sink_g)).  `sink`: float32 [Hq] or
+    None; `talk`: float32 [Hq, Hq] or None (no mixing).  `batch`: the step's descriptor (positions, sequence of each
+    token, the longest sequence).  float32 arithmetic.  Returns [T, Hq * hd] in the type of `q`."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(q, cache, block_table, sink, talk)
+    if q.dim() != 3 or q.stride(2) != 1 or q.stride(1) != q.shape[2]:
+        raise KernelError("q must be [T, Hq, hd] with contiguous heads")
+    n_tokens, n_q, hd = q.shape
+    if cache.dim() != 4 or cache.shape[1] != 2 or cache.shape[3] % hd != 0 or not cache.is_contiguous() or cache.dtype != q.dtype:
+        raise KernelError(f"cache {tuple(cache.shape)} {cache.dtype} does not fit heads of size {hd} of {q.dtype}")
+    n_kv = cache.shape[2]
+    if n_q > MAX_TALK_HEADS or n_q % n_kv != 0:
+        raise KernelError(f"{n_q} query heads on {n_kv} key/value heads: at most {MAX_TALK_HEADS} heads, in equal groups")
+    if window is not None and window < 1:
+        raise KernelError("a window holds at least the query's own key")
+    if sink is not None and (sink.dtype != torch.float32 or sink.shape != (n_q,) or not sink.is_contiguous()):
+        raise KernelError(f"the sinks must be a contiguous float32 [{n_q}] tensor")
+    if talk is not None and (talk.dtype != torch.float32 or talk.shape != (n_q, n_q) or not talk.is_contiguous()):
+        raise KernelError(f"the heads' mixing matrix must be a contiguous float32 [{n_q}, {n_q}] tensor")
+    _i32(block_table, "block_table")
+    _i32(batch.positions, "positions")
+    _i32(batch.seq_of_token, "seq_of_token")
+    if batch.positions.numel() != n_tokens or batch.seq_of_token.numel() != n_tokens or block_table.dim() != 2:
+        raise KernelError("positions and seq_of_token must be [T], block_table [B, W]")
+    static = getattr(batch, "static", None)
+    max_keys = batch.max_kv_len if static is None else static.max_keys
+    if window is not None:
+        max_keys = min(max_keys, window)
+    n_split = max(1, -(-max_keys // TALK_SPLIT))
+    width = n_q * hd
+    stats = torch.empty(n_tokens * n_split * n_q * 2, dtype=torch.float32, device=q.device)
+    out = partial = None
+    if n_split == 1:
+        out = torch.empty((n_tokens, width), dtype=q.dtype, device=q.device)
+    else:
+        partial = torch.empty((n_split, n_tokens, width), dtype=torch.float32, device=q.device)
+    lib = _build.load("attention_talk")
+    _check(
+        lib,
+        lib.cwm_talking_attention(
+            _ptr(q), ctypes.c_long(q.stride(0) if n_tokens > 1 else width), _ptr(out), _ptr(partial), _ptr(stats), _ptr(cache),
+            ctypes.c_int(_code(q.dtype)), _ptr(block_table), ctypes.c_int(block_table.shape[1]), _ptr(batch.positions),
+            _ptr(batch.seq_of_token), ctypes.c_int(n_tokens), ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(hd),
+            ctypes.c_int(cache.shape[3] // hd), ctypes.c_int(cache.shape[0]), ctypes.c_int(-1 if window is None else window - 1),
+            ctypes.c_float(scale), _ptr(sink), _ptr(talk), ctypes.c_int(n_split), _stream(),
+        ),
+    )
+    if out is not None:
+        return out
+    from . import sum_partials
+
+    return sum_partials(partial, q.dtype)
+
+
+GLA_THREADS = 256  # csrc/linear_attention.hip: threads of a walking block
+GLA_ROWS = 32  # and the rows of a column of the state that one of them holds at most
+
+
+def gla_split(dim: int) -> int:
+    """Lanes that share a column of a head's state: the fewest (1, 2, 4, 8) that leave a lane at most GLA_ROWS rows."""
+    split = 1
+    while split < 8 and -(-dim // split) > GLA_ROWS:
+        split *= 2
+    return split
+
+
+def gla_state_elems(heads: int, dim: int, vdim: int) -> int:
+    """float32 elements of one request's state of a gated linear attention, in the walking kernel's own order: per
+    (head, tile of value columns) the rows a thread holds, [row][thread]."""
+    split = gla_split(dim)
+    rows, cols = -(-dim // split), GLA_THREADS // split
+    return heads * -(-vdim // cols) * rows * GLA_THREADS
+
+
+def gla_state_unpack(flat: torch.Tensor, heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """S [heads, dim, vdim] of one request's state row (tests read states this way)."""
+    split = gla_split(dim)
+    rows, cols = -(-dim // split), GLA_THREADS // split
+    n_vt = -(-vdim // cols)
+    # [head][tile][row r][column][part]: element (d = part + split * r, e = tile * cols + column)
+    t = flat[: heads * n_vt * rows * GLA_THREADS].reshape(heads, n_vt, rows, cols, split)
+    s = t.permute(0, 2, 4, 1, 3).reshape(heads, rows * split, n_vt * cols)
+    return s[:, :dim, :vdim]
+
+
+def gated_linear_attention(
+    proj: torch.Tensor, decay_logits: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, batch: Any,
+    heads: int, dim: int, vdim: int, tau: float, eps: float, q_scale: Optional[float] = None,
+) -> torch.Tensor:
+    """Gated linear attention over the step's tokens (`csrc/linear_attention.hip`).  `proj` [T, heads * (2 dim + 2 vdim)]
+    holds queries and keys (heads * dim each), then values and the output gate's projection (heads * vdim each);
+    `decay_logits` float32 [T, heads * dim] (bias included): a key channel decays by sigmoid(logit)^(1 / tau); `weight`
+    float32 [vdim]; `state` float32 [slots, >= gla_state_elems], read and written at the sequences' slots.  Queries are
+    multiplied by `q_scale` (default dim ** -0.5).  Returns [T, heads * vdim] in proj's type: every head's result over
+    its root mean square, times weight, times silu(gate)."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(proj, decay_logits, weight, state)
+    n_tokens = proj.shape[0]
+    width = heads * (2 * dim + 2 * vdim)
+    if proj.dim() != 2 or proj.stride(1) != 1 or proj.shape[1] < width or n_tokens != batch.n_tokens:
+        raise KernelError(f"the projection {tuple(proj.shape)} must be [{batch.n_tokens}, >= {width}] with contiguous rows")
+    if decay_logits.dtype != torch.float32 or tuple(decay_logits.shape) != (n_tokens, heads * dim) or decay_logits.stride(1) != 1:
+        raise KernelError(f"the decays' logits must be float32 [{n_tokens}, {heads * dim}]")
+    if weight.dtype != torch.float32 or weight.shape != (vdim,) or not weight.is_contiguous():
+        raise KernelError(f"the weight must be a contiguous float32 [{vdim}]")
+    if dim > MAX_GLA_DIM:
+        raise KernelError(f"heads of {dim} rows: the walking kernel takes up to {MAX_GLA_DIM}")
+    need = gla_state_elems(heads, dim, vdim)
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] < need or not state.is_contiguous():
+        raise KernelError(f"the state must be a contiguous float32 [slots, >= {need}] tensor")
+    o_raw = torch.empty((n_tokens, heads * vdim), dtype=torch.float32, device=proj.device)
+    out = torch.empty((n_tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
+    lib = _build.load("linear_attention")
+    _check(
+        lib,
+        lib.cwm_gated_linear_attention(
+            _ptr(proj), ctypes.c_long(proj.stride(0) if n_tokens > 1 else proj.shape[1]), ctypes.c_int(_code(proj.dtype)),
+            _ptr(decay_logits), ctypes.c_long(decay_logits.stride(0) if n_tokens > 1 else heads * dim), _ptr(weight), _ptr(o_raw), _ptr(out),
+            _ptr(state), ctypes.c_long(state.shape[1]), _ptr(batch.state_slots), _ptr(batch.cu_q), ctypes.c_int(state.shape[0]),
+            ctypes.c_int(n_tokens), ctypes.c_int(batch.n_seqs), ctypes.c_int(heads), ctypes.c_int(dim), ctypes.c_int(vdim),
+            ctypes.c_float(tau), ctypes.c_float(eps), ctypes.c_float(dim ** -0.5 if q_scale is None else q_scale), _stream(),
+        ),
+    )
+    return out
+
+
+def short_conv(
+    x: torch.Tensor, weights: Sequence[torch.Tensor], state: Optional[torch.Tensor], batch: Any, write_state: bool = True,
+) -> Tuple[torch.Tensor, ...]:
+    """x + (causal convolution of x over each sequence of the step), a channel at a time, once for each of the one or
+    two `weights` (float32 [taps, D], a row a tap, the last row the current token's): `x` [T, D] (rows may lie apart).
+    A sequence's last taps - 1 inputs live in its row of `state` (float32 [slots, >= (taps - 1) * D], oldest first):
+    read by the portion's first tokens, then replaced (`write_state`).  Returns a [T, D] tensor of x's type a weight."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(x, state, *weights)
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[0] != batch.n_tokens:
+        raise KernelError(f"x must be [{batch.n_tokens}, D] with contiguous rows")
+    n_tokens, dim = x.shape
+    if not 1 <= len(weights) <= 2:
+        raise KernelError("one or two convolutions of the same input are taken")
+    taps = weights[0].shape[0]
+    for w in weights:
+        if w.dtype != torch.float32 or tuple(w.shape) != (taps, dim) or not w.is_contiguous():
+            raise KernelError(f"a convolution's weight must be a contiguous float32 [{taps}, {dim}] tensor (a row a tap)")
+    if not 1 <= taps <= MAX_SHORT_CONV_TAPS:
+        raise KernelError(f"{taps} taps are outside 1..{MAX_SHORT_CONV_TAPS}")
+    if taps > 1 and (state is None or state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] < (taps - 1) * dim or not state.is_contiguous()):
+        raise KernelError(f"the state must be a contiguous float32 [slots, >= {(taps - 1) * dim}] tensor")
+    outs = tuple(torch.empty((n_tokens, dim), dtype=x.dtype, device=x.device) for _ in weights)
+    lib = _build.load("short_conv")
+    _check(
+        lib,
+        lib.cwm_short_conv(
+            _ptr(x), ctypes.c_long(x.stride(0) if n_tokens > 1 else dim), ctypes.c_int(_code(x.dtype)), _ptr(weights[0]),
+            _ptr(weights[1] if len(weights) > 1 else None), _ptr(outs[0]), _ptr(outs[1] if len(weights) > 1 else None),
+            _ptr(state if taps > 1 else None), ctypes.c_long(state.shape[1] if taps > 1 else 0), _ptr(batch.state_slots), _ptr(batch.cu_q),
+            _ptr(batch.seq_of_token), ctypes.c_int(state.shape[0] if taps > 1 else 0), ctypes.c_int(n_tokens), ctypes.c_int(batch.n_seqs),
+            ctypes.c_int(dim), ctypes.c_int(taps), ctypes.c_int(int(write_state)), _stream(),
+        ),
+    )
+    return outs
+
+
+def token_side(
+    h: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, column0: int, w_gate: torch.Tensor, w_proj: torch.Tensor,
+    weight: torch.Tensor, eps: float, round_inputs: bool,
+) -> None:
+    """h (float32 [T, D]) += rms(y) * weight with y = w_proj (gelu_tanh(w_gate h) * e), e the columns column0 ..
+    column0 + side_dim of the token's row of `table` ([vocab, n]); w_gate [side_dim, D], w_proj [D, side_dim] and the
+    table have one type; `weight` float32 [D].  `round_inputs`: h and the gated values are rounded to bfloat16 where
+    they enter the two products.  float32 sums, activation and norm."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(h, tokens, table, w_gate, w_proj, weight)
+    if h.dtype != torch.float32 or h.dim() != 2 or not h.is_contiguous():
+        raise KernelError("the residual stream must be a contiguous float32 [T, D] tensor")
+    n_tokens, dim = h.shape
+    _i32(tokens, "tokens")
+    if tokens.numel() != n_tokens:
+        raise KernelError("one token per row is needed")
+    if w_gate.dim() != 2 or w_gate.shape[1] != dim or not w_gate.is_contiguous():
+        raise KernelError(f"the gate's weight must be a contiguous [side_dim, {dim}] tensor")
+    side_dim = w_gate.shape[0]
+    if tuple(w_proj.shape) != (dim, side_dim) or not w_proj.is_contiguous():
+        raise KernelError(f"the projection's weight must be a contiguous [{dim}, {side_dim}] tensor")
+    if table.dim() != 2 or table.stride(1) != 1 or column0 < 0 or column0 + side_dim > table.shape[1]:
+        raise KernelError(f"the table {tuple(table.shape)} has no columns {column0}..{column0 + side_dim - 1}")
+    if not (table.dtype == w_gate.dtype == w_proj.dtype):
+        raise KernelError("the table and the two weights must have one type")
+    if weight.dtype != torch.float32 or weight.shape != (dim,) or not weight.is_contiguous():
+        raise KernelError(f"the norm's weight must be a contiguous float32 [{dim}] tensor")
+    if side_dim > MAX_SIDE_DIM:
+        raise KernelError(f"{side_dim} side values: the kernel takes up to {MAX_SIDE_DIM}")
+    lib = _build.load("token_side")
+    _check(
+        lib,
+        lib.cwm_token_side(
+            _ptr(h), _ptr(tokens), _ptr(table), ctypes.c_long(table.stride(0)), ctypes.c_int(column0), _ptr(w_gate), _ptr(w_proj),
+            ctypes.c_int(_code(table.dtype)), _ptr(weight), ctypes.c_int(n_tokens), ctypes.c_int(dim), ctypes.c_int(side_dim),
+            ctypes.c_int(table.shape[0]), ctypes.c_float(eps), ctypes.c_int(int(round_inputs)), _stream(),
+        ),
+    )
+
+
+def gated_act_rows(x: torch.Tensor, hidden: int, activation: Any, out_dtype: torch.dtype, row_gate_col: Optional[int] = None) -> torch.Tensor:
+    """What a gated feed-forward makes of its joined product `x` ([T, >= 2 hidden] with a row's gate values first, then
+    its up values; or float32 partial sums [P, T, n], added in order first): `activation` is an `ops.GatedActivation`.
+    With `row_gate_col` every row is also multiplied by the sigmoid of that column of x.  float32 arithmetic, rounded
+    once; returns [T, hidden] of `out_dtype`."""
+    KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
+    _need_gpu(x)
+    if x.dim() == 3:
+        if x.dtype != torch.float32 or not x.is_contiguous():
+            raise KernelError("partial sums must be a contiguous float32 [P, T, n] tensor")
+        n_partials, n_rows, n = x.shape
+        ld, partial_stride = n, n_rows * n
+    elif x.dim() == 2 and x.stride(1) == 1:
+        n_partials, (n_rows, n) = 1, x.shape
+        ld, partial_stride = (x.stride(0) if n_rows > 1 else n), 0
+    else:
+        raise KernelError("gated_act_rows takes [T, n] with contiguous rows or float32 partial sums [P, T, n]")
+    if n < 2 * hidden or (row_gate_col is not None and not 0 <= row_gate_col < n):
+        raise KernelError(f"rows of {n} values do not hold a gate and an up part of {hidden} each (and the row's gate)")
+    out = torch.empty((n_rows, hidden), dtype=out_dtype, device=x.device)
+    lib = _build.load("rowwise")
+    _check(
+        lib,
+        lib.cwm_gated_act_rows(
+            _ptr(out), ctypes.c_int(_code(out_dtype)), _ptr(x), ctypes.c_int(_code(x.dtype)), ctypes.c_long(ld), ctypes.c_int(n_partials),
+            ctypes.c_long(partial_stride), ctypes.c_int(n_rows), ctypes.c_int(hidden), ctypes.c_int(-1 if row_gate_col is None else row_gate_col),
+            ctypes.c_int(activation.code()), ctypes.c_float(activation.alpha), ctypes.c_float(activation.limit), _stream(),
+        ),
+    )
+    return out

@@ -263,6 +263,155 @@ class SinkAttention(Mixer):
 register_part("mixer", "sink_attention", SinkAttention)
 
 
+class TalkingAttention(Mixer):
+    """Grouped-query attention over a paged cache whose heads exchange their softmax weights, with biased projections,
+    a sliding window and a sink in every head's softmax.
+
+        q = W_q x + b_q, k = W_k x + b_k, v = W_v x + b_v        `n_heads` heads of `qk_dim`, `n_kv_heads` of `qk_dim` (keys)
+                                                                 and `v_dim` (values); biases where `bias`
+        rotation of q and k by the position encoding             its table may turn fewer than qk_dim dimensions, in
+                                                                 adjacent pairs or in halves of the turned part
+        p_g(j) = exp(scale q_g . k_j) / (sum_i exp(scale q_g . k_i) + exp(sink_g))    over the `window` keys up to the query's own
+        w_h(j) = sum_g talk[h, g] p_g(j)                         where `talk`: the heads' weights mixed after the softmax
+        out = W_o [sum_j w_h(j) v_j of every head, from h's own key/value head] + b_o
+
+    The sink (where `sink`) has no key and no value, is not scaled, counts once and is not mixed.  With
+    `own_kv=False` the mixer has no key and value projections: it is run on a cache that another layer of equal
+    key/value heads, sizes and rotation has written in the same step (`write_cache` false).  `cache_window` is what
+    the cache keeps (default: `window`): a layer whose cache another layer reads through a longer window keeps that
+    longer one.  Keys and values are cached with one head size, the larger of qk_dim and v_dim rounded up to a
+    multiple of 16 (zeros beyond a head's own size; W_o is widened by zero columns at load).  Without `talk` the
+    paged attention kernels of the other mixers serve it.  `names`: the tensors' local names for the roles q, k, v,
+    o, q_bias, k_bias, v_bias, o_bias, sink and talk."""
+
+    replayable = True
+    DEFAULT_NAMES = {
+        "q": "q", "k": "k", "v": "v", "o": "o", "q_bias": "q.b", "k_bias": "k.b", "v_bias": "v.b", "o_bias": "o.b",
+        "sink": "sink", "talk": "talk",
+    }
+    _KEEP_WINDOW = object()
+
+    def __init__(
+        self,
+        dim: int,
+        n_heads: int,
+        n_kv_heads: int,
+        qk_dim: int,
+        v_dim: int,
+        scale: float,
+        window: Optional[int] = None,
+        cache_window: Any = _KEEP_WINDOW,
+        bias: bool = True,
+        sink: bool = True,
+        talk: bool = True,
+        own_kv: bool = True,
+        position_encoding: Optional[PartChoice] = None,
+        names: Optional[Mapping[str, str]] = None,
+    ) -> None:
+        if n_heads % n_kv_heads != 0:
+            raise ValueError(f"{n_heads} query heads do not divide into {n_kv_heads} key/value heads")
+        head_dim = -(-max(qk_dim, v_dim) // 16) * 16
+        if min(qk_dim, v_dim) < 1 or head_dim > MAX_HEAD_DIM:
+            raise ValueError(f"heads of {qk_dim} (queries, keys) and {v_dim} (values) are outside 1..{MAX_HEAD_DIM}, the sizes the attention kernels take")
+        if window is not None and window < 1:
+            raise ValueError("a window holds at least the query's own key")
+        if talk and n_heads > ops.MAX_TALK_HEADS:
+            raise ValueError(f"{n_heads} heads that mix their weights: the kernel takes up to {ops.MAX_TALK_HEADS}")
+        self.dim, self.n_heads, self.n_kv_heads = dim, n_heads, n_kv_heads
+        self.qk_dim, self.v_dim, self.head_dim = qk_dim, v_dim, head_dim
+        self.scale, self.window = float(scale), window
+        self.cache_window = window if cache_window is self._KEEP_WINDOW else cache_window
+        if self.cache_window is not None and (window is None or self.cache_window < window):
+            raise ValueError("the cache must keep at least the keys of the mixer's own window")
+        self.bias, self.sink, self.talk, self.own_kv = bias, sink, talk, own_kv
+        self.names = {**self.DEFAULT_NAMES, **dict(names or {})}
+        self.position_encoding: Optional[PositionEncoding] = (
+            position_encoding.build("position_encoding") if position_encoding is not None else None
+        )
+
+    def cache_spec(self) -> PagedKVSpec:
+        return PagedKVSpec(n_kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.cache_window)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n = self.names
+        q_out, k_out, v_out = self.n_heads * self.qk_dim, self.n_kv_heads * self.qk_dim, self.n_kv_heads * self.v_dim
+        specs = {n["q"]: TensorSpec((q_out, self.dim)), n["o"]: TensorSpec((self.dim, self.n_heads * self.v_dim))}
+        if self.own_kv:
+            specs[n["k"]] = TensorSpec((k_out, self.dim))
+            specs[n["v"]] = TensorSpec((v_out, self.dim))
+        if self.bias:
+            specs[n["q_bias"]] = TensorSpec((q_out,), precision="stored")
+            specs[n["o_bias"]] = TensorSpec((self.dim,), precision="stored")
+            if self.own_kv:
+                specs[n["k_bias"]] = TensorSpec((k_out,), precision="stored")
+                specs[n["v_bias"]] = TensorSpec((v_out,), precision="stored")
+        if self.sink:
+            specs[n["sink"]] = TensorSpec((self.n_heads,), init="zeros", precision="stored")
+        if self.talk:
+            specs[n["talk"]] = TensorSpec((self.n_heads, self.n_heads), init="identity", precision="stored")
+        return specs
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        n = self.names
+        roles = ("q", "k", "v") if self.own_kv else ("q",)
+        weights = {r: tensors[n[r]] for r in roles}
+        biases = {r: (tensors[n[r + "_bias"]].float() if self.bias else None) for r in roles}
+        device = weights["q"].device
+        self.table: Optional[torch.Tensor] = None
+        if self.position_encoding is not None:
+            self.position_encoding.bind({}, runtime)
+            table = self.position_encoding.rotary_table()
+            if table is not None:
+                turned = 2 * table.numel()
+                if turned > self.qk_dim:
+                    raise ValueError(f"{turned} rotated dimensions exceed the head's {self.qk_dim}")
+                if self.position_encoding.rotary_pairing() == "halves":
+                    # the kernels turn adjacent elements: bring element i and i + turned / 2 of every query and key head
+                    # side by side, once, by the order of the projections' rows (a layer that reads another's cache
+                    # turns with the same table, so its queries meet that layer's keys in the same order)
+                    half = turned // 2
+                    order = torch.cat([torch.stack([torch.arange(half), torch.arange(half) + half], dim=1).reshape(-1), torch.arange(turned, self.qk_dim)]).to(device)
+                    for r, heads in (("q", self.n_heads), ("k", self.n_kv_heads)):
+                        if r not in weights:
+                            continue
+                        rows = (torch.arange(heads, device=device)[:, None] * self.qk_dim + order[None, :]).reshape(-1)
+                        weights[r] = weights[r][rows]
+                        if biases[r] is not None:
+                            biases[r] = biases[r][rows]
+                # a frequency of 0 leaves its pair alone: the head's other dimensions, and the padding
+                self.table = torch.zeros(self.head_dim // 2, dtype=torch.float32, device=device)
+                self.table[: table.numel()] = table.to(device)
+        self.proj = LinearWeights.joined([weights[r] for r in roles], [biases[r] for r in roles], stream_copy=runtime.stream_copies)
+        wo = tensors[n["o"]]
+        if self.v_dim != self.head_dim:
+            # the attention kernels return heads of the cached size: columns of zeros where a head's values end
+            wide = torch.zeros((self.dim, self.n_heads, self.head_dim), dtype=wo.dtype, device=device)
+            wide[:, :, : self.v_dim] = wo.reshape(self.dim, self.n_heads, self.v_dim)
+            wo = wide.reshape(self.dim, self.n_heads * self.head_dim)
+        self.wo = LinearWeights(wo, tensors[n["o_bias"]].float() if self.bias else None, stream_copy=runtime.stream_copies)
+        self.sinks = tensors[n["sink"]].float().contiguous() if self.sink else None
+        self.talk_matrix = tensors[n["talk"]].float().contiguous() if self.talk else None
+
+    def forward(self, x: torch.Tensor, batch: Any, cache: Any, write_cache: bool = True) -> torch.Tensor:
+        if write_cache != self.own_kv:
+            raise ValueError("a mixer with key and value projections writes its cache, one without reads another layer's")
+        proj = self.proj(x)
+        q = ops.qk_norm_rope_write(
+            proj, self.n_heads, self.n_kv_heads if self.own_kv else 0, self.qk_dim, self.v_dim, self.head_dim, None, None, 1.0,
+            batch.positions, self.table, self.runtime.act_dtype,
+            cache.cache if write_cache else None, cache.block_table if write_cache else None, batch.seq_of_token if write_cache else None,
+        )
+        if self.talk_matrix is not None:
+            attn = ops.talking_attention(q, cache.cache, cache.block_table, batch, self.window, self.scale, sink=self.sinks, talk=self.talk_matrix)
+        else:
+            attn = ops.paged_attention(q, cache.cache, cache.block_table, batch, self.window, self.scale, sink=self.sinks)
+        return self.wo(attn, partials_ok=self.wo.bias is None)  # added into the residual by the next norm
+
+
+register_part("mixer", "talking_attention", TalkingAttention)
+
+
 class HeadNormAttention(Mixer):
     """Grouped-query attention over a paged cache with a norm of every query and key head, a cap on the scores, an
     output gate, and optionally values blended with those of an earlier layer.

@@ -13,7 +13,11 @@ Kinds of part and their registries (name -> class):
   BLOCKS              arrangement of the above in one layer
   EMBEDDINGS          token ids (and whatever else of the step) -> the float32 residual stream
   CONNECTIONS         how a sublayer reads the residual and how its result goes back into it
+  TOKEN_INPUTS        what a layer adds to the residual from the step's tokens themselves
   HEADS               normalised rows -> float32 logits
+
+A tensor name that a part declares with a leading "/" is the tensor's full name in the model folder: no layer's
+and no role's prefix goes before it, so parts of several layers can read one tensor, which is loaded once.
 """
 
 from __future__ import annotations
@@ -37,6 +41,18 @@ class TensorSpec:
     # reference casts every parameter, cwm/model/parallelize_transformer.py:50-59); "stored" keeps a
     # tensor that is stored in 32 bits in float32 (norm weights, tables whose precision matters)
     precision: str = "activation"
+    # a tensor that a folder may hold or not: the loader passes it on where it is there and does not miss it where
+    # it is not (the part that names it must do without)
+    optional: bool = False
+
+    # A size written as a negative number is free: the folder's tensor decides it (a low rank that no key of the
+    # configuration names), and the part reads it from the tensor it is given.  Its magnitude is the size that random
+    # weights are drawn with.
+    def drawn_shape(self) -> Tuple[int, ...]:
+        return tuple(abs(n) for n in self.shape)
+
+    def fits(self, shape: Tuple[int, ...]) -> bool:
+        return len(shape) == len(self.shape) and all(n < 0 or n == m for n, m in zip(self.shape, shape))
 
 
 # --------------------------------------------------------------------------- #
@@ -243,6 +259,20 @@ class Connection(Part):
         raise NotImplementedError
 
 
+class TokenInput(Part):
+    """What a layer adds to the residual from the step's tokens themselves (a second embedding of the token that
+    every layer reads its own part of, say)."""
+
+    def forward(self, h: torch.Tensor, batch: Any) -> None:
+        """`h` is the float32 residual [T, D] with every pending update already in it; the part adds into it in place."""
+        raise NotImplementedError
+
+
+def is_absolute(name: str) -> bool:
+    """Whether a declared tensor name is the tensor's full name in the model folder."""
+    return name.startswith("/")
+
+
 class Block(Part):
     """One layer: an arrangement of any number of norms, mixers and feed-forwards.
 
@@ -275,14 +305,16 @@ class Block(Part):
         specs: Dict[str, TensorSpec] = {}
         for role, part in self._own_parts().items():
             for name, spec in part.tensor_specs().items():
-                specs[self.names[role] + name] = spec
+                specs[name if is_absolute(name) else self.names[role] + name] = spec
         return specs
 
     def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
         super().bind(tensors, runtime)
         for role, part in self._own_parts().items():
             prefix = self.names[role]
-            part.bind({n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}, runtime)
+            own = {n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix) and not is_absolute(n)}
+            own.update({n: tensors[n] for n in part.tensor_specs() if is_absolute(n)})
+            part.bind(own, runtime)
 
     def mixers(self) -> List[Mixer]:
         """The block's mixers in the order in which `forward` gets their caches: each has a cache slot of its
@@ -319,6 +351,7 @@ BLOCKS: Dict[str, Callable[..., Block]] = {}
 EMBEDDINGS: Dict[str, Callable[..., Embedding]] = {}
 HEADS: Dict[str, Callable[..., Head]] = {}
 CONNECTIONS: Dict[str, Callable[..., Connection]] = {}
+TOKEN_INPUTS: Dict[str, Callable[..., TokenInput]] = {}
 
 _REGISTRIES = {
     "norm": NORMS,
@@ -329,12 +362,14 @@ _REGISTRIES = {
     "embedding": EMBEDDINGS,
     "head": HEADS,
     "connection": CONNECTIONS,
+    "token_input": TOKEN_INPUTS,
 }
 
 
 def register_part(kind: str, name: str, factory: Callable[..., Part]) -> None:
     """Make `factory` available to architecture builders as part `name` of `kind`
-    ("norm", "mixer", "feed_forward", "position_encoding", "block", "embedding", "head" or "connection")."""
+    ("norm", "mixer", "feed_forward", "position_encoding", "block", "embedding", "head", "connection" or
+    "token_input")."""
     if kind not in _REGISTRIES:
         raise KeyError(f"unknown kind of part {kind!r}; kinds: {', '.join(_REGISTRIES)}")
     _REGISTRIES[kind][name] = factory
@@ -413,10 +448,14 @@ class LayerPlan:
 class LayerCall:
     """One entry of the run order.  `layer` indexes `ModelPlan.layers`; a layer may
     be named more than once.  `cache_of` names an earlier entry of the run order
-    whose cache this call reads instead of keeping one of its own."""
+    whose cache this call reads instead of keeping one of its own.  `shared_mixers` narrows that to some of the
+    block's mixers (indices into `Block.mixers()`; the earlier entry's mixer of the same index owns the cache):
+    the others keep caches of their own, and the block's `forward` is then told mixer by mixer which ones
+    write (a tuple of booleans in the place of `write_cache`)."""
 
     layer: int
     cache_of: Optional[int] = None
+    shared_mixers: Optional[Tuple[int, ...]] = None
 
 
 @dataclass(frozen=True)

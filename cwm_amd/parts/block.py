@@ -6,7 +6,7 @@ from typing import Any, Mapping, Optional
 
 import torch
 
-from .base import Block, Connection, FeedForward, Mixer, Norm, register_part
+from .base import Block, Connection, FeedForward, Mixer, Norm, TokenInput, register_part
 
 
 class PreNormBlock(Block):
@@ -155,3 +155,63 @@ class ParallelPreNormBlock(Block):
 
 
 register_part("block", "parallel_pre_norm", ParallelPreNormBlock)
+
+
+class SharedNormParallelBlock(Block):
+    """h += mixer(u_1) + feed_forward(u_2), where both sublayers read one norm of the residual, n = norm(h): u_1 = u_2 = n,
+    or, with `conv` (a mixer with a state of its own that makes one input a sublayer from n: short convolutions over
+    time), u_1, u_2 = conv(n).  With `token_input` the layer then adds its own input from the step's tokens, which
+    reads the residual after the sublayers' sum: the block then does that sum itself (one kernel, float32, the
+    sublayers' results in their order) and leaves no pending update; without one the sum is left to the norm that
+    reads the residual next, as in `ParallelPreNormBlock`.  A layer without a feed-forward names none.
+
+    The block's mixers, in the order of their caches: `conv` where there is one, then the mixer (or its children).
+    A run-order entry may let the mixer read another entry's cache while the convolution keeps a state of its own:
+    `write_cache` is then a tuple, one boolean a mixer."""
+
+    def __init__(
+        self, names: Mapping[str, str], norm: Norm, mixer: Mixer, conv: Optional[Mixer] = None,
+        feed_forward: Optional[FeedForward] = None, token_input: Optional[TokenInput] = None,
+    ) -> None:
+        parts = dict(norm=norm)
+        if conv is not None:
+            parts["conv"] = conv
+        parts["mixer"] = mixer
+        if feed_forward is not None:
+            parts["feed_forward"] = feed_forward
+        if token_input is not None:
+            parts["token_input"] = token_input
+        super().__init__(names, **parts)
+        self.norm, self.conv, self.mixer, self.feed_forward, self.token_input = norm, conv, mixer, feed_forward, token_input
+
+    def mixers(self):
+        children = getattr(self.mixer, "children", None)
+        own = list(children()) if children is not None else [self.mixer]
+        return ([self.conv] if self.conv is not None else []) + own
+
+    def forward(self, h: torch.Tensor, delta: Any, batch: Any, cache: Any, write_cache: Any = True) -> Any:
+        from .. import ops
+
+        views = cache if isinstance(cache, tuple) else ((cache,) if len(self.mixers()) == 1 else ())
+        writes = tuple(write_cache) if isinstance(write_cache, tuple) else (write_cache,) * len(views)
+        x = self.norm.forward(h, delta)
+        x1 = x2 = x
+        if self.conv is not None:
+            made = self.conv.forward(x, batch, views[0], writes[0])
+            x1, x2 = made[0], made[-1]
+            views, writes = views[1:], writes[1:]
+        if len(set(writes)) > 1:
+            raise ValueError("the mixers side by side of one layer all write their caches or all read another layer's")
+        mixed = self.mixer.forward(x1, batch, views[0] if len(views) == 1 else views, writes[0])
+        terms = list(mixed.terms) if isinstance(mixed, ops.ScaledSum) else [(mixed, 1.0)]
+        if self.feed_forward is not None:
+            out = self.feed_forward.forward(x2, batch)
+            terms.extend(out.terms if isinstance(out, ops.ScaledSum) else [(out, 1.0)])
+        if self.token_input is None:
+            return ops.ScaledSum(terms)
+        ops.add_layernorm(h, ops.ScaledSum(terms), None, None, 1.0, self.runtime.act_dtype)  # the sum alone
+        self.token_input.forward(h, batch)
+        return None
+
+
+register_part("block", "shared_norm_parallel", SharedNormParallelBlock)

@@ -149,3 +149,79 @@ class MatrixMemory(Mixer):
 
 
 register_part("mixer", "matrix_memory", MatrixMemory)
+
+
+class GatedLinearAttention(Mixer):
+    """Linear attention with a decay per key channel, with a per-request state.  q = W_q x * head_dim^(-1/2), k = W_k x
+    (heads x head_dim), v = W_v x (heads x v_dim); per head
+        alpha_t = sigmoid(W_a2 (W_a1 x) + b_a)^(1 / tau)                a decay a key channel, through a low rank
+        S_t = diag(alpha_t) S_(t-1) + k_t v_t^T,      y_t = S_t^T q_t
+    with S zero at a request's start; then out = W_o (y / rms(y per head) * weight * silu(W_g x)), the weight of v_dim
+    values shared by the heads.  The decays' second projection leaves its product in float32, and decays, state, the
+    result's norm and its gate are float32 whatever the activation type.  A request's state is one float32 row in the
+    walking kernel's own layout (`ops.gla_state_elems`).  `names`: local names of the tensors for the roles q, k, v, g,
+    o, norm, a1, a2, a2_bias.  `decay_rank` None: the rank is whatever the folder's a1 and a2 have (random weights are
+    drawn with `DRAWN_RANK`)."""
+
+    replayable = True
+    DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "norm": "norm", "a1": "a1", "a2": "a2", "a2_bias": "a2.b"}
+    DRAWN_RANK = 16
+
+    def __init__(
+        self, dim: int, heads: int, head_dim: int, v_dim: int, tau: float, decay_rank: Optional[int], eps: float,
+        names: Optional[Mapping[str, str]] = None,
+    ) -> None:
+        if min(heads, head_dim, v_dim, decay_rank or 1) < 1 or head_dim > ops.MAX_GLA_DIM:
+            raise ValueError(f"heads of {head_dim} x {v_dim}: the walking kernel takes 1..{ops.MAX_GLA_DIM} rows")
+        if not tau > 0:
+            raise ValueError("tau must be positive")
+        self.dim, self.heads, self.head_dim, self.v_dim, self.decay_rank = dim, heads, head_dim, v_dim, decay_rank
+        self.tau, self.eps = float(tau), float(eps)
+        self.names = {**self.DEFAULT_NAMES, **dict(names or {})}
+        self._state_elems: Optional[int] = None
+
+    @property
+    def state_elems(self) -> int:
+        if self._state_elems is None:
+            self._state_elems = ops.gla_state_elems(self.heads, self.head_dim, self.v_dim)
+        return self._state_elems
+
+    def cache_spec(self) -> StateSpec:
+        return StateSpec((self.state_elems,), torch.float32)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n = self.names
+        qk, vv = self.heads * self.head_dim, self.heads * self.v_dim
+        return {
+            n["q"]: TensorSpec((qk, self.dim)),
+            n["k"]: TensorSpec((qk, self.dim)),
+            n["v"]: TensorSpec((vv, self.dim)),
+            n["g"]: TensorSpec((vv, self.dim)),
+            n["o"]: TensorSpec((self.dim, vv)),
+            n["norm"]: TensorSpec((self.v_dim,), init="norm", precision="stored"),
+            n["a1"]: TensorSpec((self.decay_rank or -self.DRAWN_RANK, self.dim)),
+            n["a2"]: TensorSpec((qk, self.decay_rank or -self.DRAWN_RANK)),
+            n["a2_bias"]: TensorSpec((qk,), precision="stored"),
+        }
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        n = self.names
+        if tensors[n["a1"]].shape[0] != tensors[n["a2"]].shape[1]:
+            raise ValueError(f"the decays' two projections do not meet: {tuple(tensors[n['a1']].shape)} and {tuple(tensors[n['a2']].shape)}")
+        self.proj = LinearWeights.joined([tensors[n[r]] for r in ("q", "k", "v", "g", "a1")], [None] * 5, stream_copy=runtime.stream_copies)
+        self.width = 2 * self.heads * (self.head_dim + self.v_dim)
+        self.decay_up = LinearWeights(tensors[n["a2"]], tensors[n["a2_bias"]].float())
+        self.w_out = LinearWeights(tensors[n["o"]], stream_copy=runtime.stream_copies)
+        self.weight = tensors[n["norm"]].float().contiguous()
+
+    def forward(self, x: torch.Tensor, batch: Any, cache: Any, write_cache: bool = True) -> torch.Tensor:
+        if not write_cache:
+            raise ValueError("a linear attention cannot read another layer's state")
+        proj = self.proj(x)
+        logits = self.decay_up(proj[:, self.width :], out_dtype=torch.float32)  # float32 sums, not rounded: they enter the recurrence
+        y = ops.gated_linear_attention(proj, logits, self.weight, cache.state, batch, self.heads, self.head_dim, self.v_dim, self.tau, self.eps)
+        return self.w_out(y, partials_ok=True)
+
+
+register_part("mixer", "gated_linear_attention", GatedLinearAttention)

@@ -87,12 +87,12 @@ def load_tensors(
                 shapes[name] = tuple(sl.get_shape())
                 stored[name] = str(sl.get_dtype())
 
-    missing = sorted(set(specs) - set(where))
+    missing = sorted(name for name in set(specs) - set(where) if not specs[name].optional)
     unexpected = sorted(set(where) - set(specs))
     wrong = [
         f"{name}: expected {tuple(specs[name].shape)}, found {shapes[name]}"
         for name in sorted(set(specs) & set(where))
-        if tuple(specs[name].shape) != shapes[name]
+        if not specs[name].fits(shapes[name])
     ]
     if missing or unexpected or wrong or duplicates:
         lines = [f"the tensors in {folder} do not fit the model:"]

@@ -38,23 +38,24 @@ def random_tensor(
 ) -> torch.Tensor:
     gen = torch.Generator(device=device)
     gen.manual_seed(_tensor_seed(seed, name))
+    shape = spec.drawn_shape()
     if spec.kind == "int":
-        return torch.zeros(spec.shape, dtype=torch.int32, device=device)
+        return torch.zeros(shape, dtype=torch.int32, device=device)
     if spec.init == "norm":
         if norm_init == "ones":
-            t = torch.ones(spec.shape, dtype=torch.float32, device=device)
+            t = torch.ones(shape, dtype=torch.float32, device=device)
         elif norm_init == "uniform":
-            t = torch.rand(spec.shape, generator=gen, dtype=torch.float32, device=device) + 0.5
+            t = torch.rand(shape, generator=gen, dtype=torch.float32, device=device) + 0.5
         else:
             raise ValueError(f"norm_init must be 'ones' or 'uniform', found {norm_init!r}")
     elif spec.init == "zeros":
-        t = torch.zeros(spec.shape, dtype=torch.float32, device=device)
+        t = torch.zeros(shape, dtype=torch.float32, device=device)
     elif spec.init == "ones":
-        t = torch.ones(spec.shape, dtype=torch.float32, device=device)
+        t = torch.ones(shape, dtype=torch.float32, device=device)
     elif spec.init == "identity":
-        t = torch.eye(spec.shape[0], spec.shape[1], dtype=torch.float32, device=device)
+        t = torch.eye(shape[0], shape[1], dtype=torch.float32, device=device)
     else:
-        t = torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * std
+        t = torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * std
     return t.to(dtype)
 
 

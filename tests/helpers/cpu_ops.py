@@ -375,6 +375,111 @@ def qk_norm_rope_write(qkv, n_q_heads, n_kv_heads, qk_dim, v_dim, head_dim, q_we
     return q
 
 
+def talking_attention(q, cache, block_table, batch, window, scale, sink=None, talk=None):
+    n_tokens, n_q, hd = q.shape
+    n_kv = cache.shape[2]
+    page_size = cache.shape[3] // hd
+    group = n_q // n_kv
+    out = torch.empty((n_tokens, n_q, hd), dtype=torch.float32)
+    for t in range(n_tokens):
+        p = int(batch.positions[t])
+        b = int(batch.seq_of_token[t])
+        lo = 0 if window is None else max(0, p - (window - 1))
+        keys, vals = [], []
+        for j in range(lo, p + 1):
+            page = int(block_table[b, j // page_size])
+            assert page >= 0, f"key {j} of sequence {b} has no page"
+            kk_, vv_ = cache_layout.read_kv(cache, page, j % page_size, hd)
+            keys.append(kk_.float())
+            vals.append(vv_.float())
+        kk = torch.stack(keys, 1)  # [n_kv, n, hd]
+        vv = torch.stack(vals, 1)
+        weights = []
+        for h in range(n_q):
+            s = (kk[h // group] @ q[t, h].float()) * scale
+            if sink is not None:
+                weights.append(torch.softmax(torch.cat([s, sink[h].float().reshape(1)]), -1)[:-1])
+            else:
+                weights.append(torch.softmax(s, -1))
+        w = torch.stack(weights)  # [n_q, n]
+        if talk is not None:
+            w = talk.float() @ w
+        for h in range(n_q):
+            out[t, h] = w[h] @ vv[h // group]
+    return out.reshape(n_tokens, n_q * hd).to(q.dtype)
+
+
+def gated_linear_attention(proj, decay_logits, weight, state, batch, heads, dim, vdim, tau, eps, q_scale=None):
+    """The state's layout is the stand-in's own: per head the matrix [dim, vdim]."""
+    n = proj.shape[0]
+    p = proj.float()
+    q = p[:, : heads * dim].reshape(n, heads, dim) * (dim ** -0.5 if q_scale is None else q_scale)
+    k = p[:, heads * dim : 2 * heads * dim].reshape(n, heads, dim)
+    v = p[:, 2 * heads * dim : 2 * heads * dim + heads * vdim].reshape(n, heads, vdim)
+    g = p[:, 2 * heads * dim + heads * vdim : 2 * heads * (dim + vdim)].reshape(n, heads, vdim)
+    alpha = torch.exp(torch.nn.functional.logsigmoid(decay_logits.float()) / tau).reshape(n, heads, dim)
+    y = torch.zeros((n, heads, vdim))
+    for b in range(batch.n_seqs):
+        row = state[int(batch.state_slots[b])]
+        S = row[: heads * dim * vdim].reshape(heads, dim, vdim).clone()
+        for t in range(int(batch.cu_q[b]), int(batch.cu_q[b + 1])):
+            S = alpha[t][:, :, None] * S + k[t][:, :, None] * v[t][:, None, :]
+            y[t] = torch.einsum("hde,hd->he", S, q[t])
+        row[: heads * dim * vdim] = S.reshape(-1)
+    y = y * torch.rsqrt((y * y).mean(-1, keepdim=True) + eps) * weight.float()
+    return (y * (g * torch.sigmoid(g))).reshape(n, heads * vdim).to(proj.dtype)
+
+
+def short_conv(x, weights, state, batch, write_state=True):
+    taps, dim = weights[0].shape
+    xf = x.float()
+    outs = [torch.empty_like(xf) for _ in weights]
+    for b in range(batch.n_seqs):
+        t0, t1 = int(batch.cu_q[b]), int(batch.cu_q[b + 1])
+        if taps > 1:
+            row = state[int(batch.state_slots[b])]
+            past = row[: (taps - 1) * dim].reshape(taps - 1, dim)
+            full = torch.cat([past, xf[t0:t1]])
+        else:
+            full = xf[t0:t1]
+        for w, out in zip(weights, outs):
+            for t in range(t1 - t0):
+                out[t0 + t] = xf[t0 + t] + (w.float() * full[t : t + taps]).sum(0)
+        if taps > 1 and write_state:
+            row[: (taps - 1) * dim] = full[full.shape[0] - (taps - 1) :].reshape(-1)
+    return tuple(out.to(x.dtype) for out in outs)
+
+
+def _as(t, dtype):
+    return t.to(dtype).float()
+
+
+def token_side(h, tokens, table, column0, w_gate, w_proj, weight, eps, round_inputs):
+    side_dim = w_gate.shape[0]
+    rd = torch.bfloat16 if round_inputs else torch.float32
+    z = _as(_as(h, rd) @ w_gate.float().T, rd)
+    gelu = 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+    g = _as(gelu * table[tokens.long(), column0 : column0 + side_dim].float(), rd)
+    y = g @ w_proj.float().T
+    h += y * torch.rsqrt((y * y).mean(-1, keepdim=True) + eps) * weight.float()
+
+
+def gated_act_rows(x, hidden, activation, out_dtype, row_gate_col=None):
+    if x.dim() == 3:
+        x = x.sum(0)
+    x = x.float()
+    g, u = x[:, :hidden], x[:, hidden : 2 * hidden]
+    if activation.kind == "clamped_swish":
+        g = torch.clamp(g, max=activation.limit)
+        u = torch.clamp(u, min=-activation.limit, max=activation.limit)
+        y = g * torch.sigmoid(activation.alpha * g) * (u + 1.0)
+    else:
+        y = g * torch.sigmoid(g) * u
+    if row_gate_col is not None:
+        y = y * torch.sigmoid(x[:, row_gate_col : row_gate_col + 1])
+    return y.to(out_dtype)
+
+
 def _total(delta):
     """A pending update (a tensor, partial sums, or a sum of scaled terms) as one float32 tensor."""
     terms = delta.terms if hasattr(delta, "terms") else [(delta, 1.0)]
@@ -468,6 +573,7 @@ def matrix_memory(proj, gates, weight, state, batch, heads, dim, vdim, cap, eps,
 
 
 STAND_INS = (
+    "talking_attention", "gated_linear_attention", "short_conv", "token_side", "gated_act_rows",
     "add_layernorm", "head_norm_rope_write", "matrix_memory",
     "embedding_streams", "stream_mix_norm", "act_rows", "qk_norm_rope_write",
     "embedding", "add_rmsnorm", "silu_mul", "gate_up_silu", "linear", "gemm_f32", "gemm_bf16",
