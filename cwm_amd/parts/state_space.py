@@ -219,7 +219,9 @@ class GatedLinearAttention(Mixer):
         if not write_cache:
             raise ValueError("a linear attention cannot read another layer's state")
         proj = self.proj(x)
-        logits = self.decay_up(proj[:, self.width :], out_dtype=torch.float32)  # float32 sums, not rounded: they enter the recurrence
+        # the low rank's second product: exact products and float32 sums, not rounded (they enter the recurrence); its K
+        # is a few tens, which the float32 kernel takes whatever the size
+        logits = ops.gemm_f32(proj[:, self.width :], self.decay_up.weight, self.decay_up.bias, torch.float32)
         y = ops.gated_linear_attention(proj, logits, self.weight, cache.state, batch, self.heads, self.head_dim, self.v_dim, self.tau, self.eps)
         return self.w_out(y, partials_ok=True)
 
