@@ -199,8 +199,20 @@ def router_logits(w: Dict[str, torch.Tensor], p: str, h: torch.Tensor) -> torch.
     return h @ w[p + "router"].T + w[p + "router.b"]
 
 
-def expert_ff(w: Dict[str, torch.Tensor], p: str, mlp: dict, h: torch.Tensor, rounded: bool = False) -> torch.Tensor:
-    chosen, weights = route(router_logits(w, p, h), mlp["router"]["top"])
+def route_margin(logits: torch.Tensor, top: int) -> torch.Tensor:
+    """How far, as a share of the largest logit's size, the last chosen logit lies above the first one left out: a
+    change of the logits by less cannot turn the choice (infinite where every expert is chosen)."""
+    if top >= logits.shape[-1]:
+        return torch.full(logits.shape[:-1], float("inf"), dtype=logits.dtype)
+    values = torch.sort(logits, dim=-1, descending=True).values
+    return (values[..., top - 1] - values[..., top]) / logits.abs().max(dim=-1).values.clamp_min(1e-30)
+
+
+def expert_ff(w: Dict[str, torch.Tensor], p: str, mlp: dict, h: torch.Tensor, rounded: bool = False, margins: Optional[list] = None) -> torch.Tensor:
+    logits = router_logits(w, p, h)
+    if margins is not None:
+        margins.append(route_margin(logits, mlp["router"]["top"]))
+    chosen, weights = route(logits, mlp["router"]["top"])
     out = torch.zeros(h.shape[0], w[p + "e0.down"].shape[0], dtype=h.dtype)
     for t in range(h.shape[0]):
         for e, c in zip(chosen[t].tolist(), weights[t]):
@@ -211,11 +223,11 @@ def expert_ff(w: Dict[str, torch.Tensor], p: str, mlp: dict, h: torch.Tensor, ro
     return out
 
 
-def feed_forward(w: Dict[str, torch.Tensor], p: str, mlp: dict, h: torch.Tensor, rounded: bool = False) -> torch.Tensor:
+def feed_forward(w: Dict[str, torch.Tensor], p: str, mlp: dict, h: torch.Tensor, rounded: bool = False, margins: Optional[list] = None) -> torch.Tensor:
     if mlp["kind"] == "dense":
         return dense_ff(w, p, mlp["limit"], h, rounded)
     if mlp["kind"] == "moe":
-        return expert_ff(w, p, mlp, h, rounded)
+        return expert_ff(w, p, mlp, h, rounded, margins)
     raise ValueError(mlp["kind"])
 
 
@@ -227,9 +239,13 @@ def token_side(w: Dict[str, torch.Tensor], p: str, x: torch.Tensor, rows: torch.
     return unit_rms(y, eps) * w[p + "norm"]
 
 
-def forward(config: dict, w: Dict[str, torch.Tensor], tokens: List[int], rounded: bool = False, layers_out: Optional[list] = None) -> torch.Tensor:
+def forward(
+    config: dict, w: Dict[str, torch.Tensor], tokens: List[int], rounded: bool = False, layers_out: Optional[list] = None,
+    margins: Optional[list] = None,
+) -> torch.Tensor:
     """Logits [T, vocab] of one whole sequence.  `rounded`: inputs of matrix products are rounded to bfloat16 where
-    an engine that stores activations in bfloat16 would.  `layers_out` receives the residual after every layer."""
+    an engine that stores activations in bfloat16 would.  `layers_out` receives the residual after every layer,
+    `margins` every router's margins [T] (see `route_margin`)."""
     rd = bf16_round if rounded else (lambda t: t)
     eps = config["norm"]["eps"]
     tok = torch.tensor(tokens, dtype=torch.long)
@@ -243,20 +259,22 @@ def forward(config: dict, w: Dict[str, torch.Tensor], tokens: List[int], rounded
         a, b = h, h
         if canon is not None:
             a = rd(h + causal_conv(h, w[p + "canon1"]))
-            b = rd(h + causal_conv(h, w[p + "canon2"]))
+            if layer.get("mlp") is not None:
+                b = rd(h + causal_conv(h, w[p + "canon2"]))
         m = layer["mixer"]
-        if layer["type"] == "attention":
+        kind = layer["type"].split("_")[0]  # a numeric suffix marks another set of sizes of the same mixer
+        if kind == "attention":
             if m.get("kv_from") is not None:
                 keys, values = cached[m["kv_from"]]
             else:
                 keys, values = attention_keys_values(w, p + "mix.", m, a, rounded)
                 cached[i] = (keys, values)
             mixed = attention_mixer(w, p + "mix.", m, a, keys, values, rounded)
-        elif layer["type"] == "gla":
+        elif kind == "gla":
             mixed = gla_mixer(w, p + "mix.", m, a, eps, rounded)
         else:
             raise ValueError(layer["type"])
-        ff = feed_forward(w, p + "mlp.", layer["mlp"], b, rounded) if layer.get("mlp") is not None else 0.0
+        ff = feed_forward(w, p + "mlp.", layer["mlp"], b, rounded, margins) if layer.get("mlp") is not None else 0.0
         x = x + (mixed + ff)
         if side is not None:
             dim = side["dim"]
