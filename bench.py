@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bf16|fp32]
     python bench.py --shape llama8b --serve 64     (requests through the scheduler instead)
-    python bench.py --compare lapevik|segedra      (another design beside the dense decoder of equal size instead)
+    python bench.py --compare lapevik|segedra|dogotar|digasun   (another design beside the dense decoder of equal size instead)
 
 Default run: the layer sizes of the CWM-32B shape with random weights, a batch of 8
 requests at a context of 32,768 tokens each; a step is one decode step of the whole
@@ -168,7 +168,7 @@ class ShapeBench:
                     self.expert_bytes.append([0, part.top, part.n_experts, layer.prefix + block.names[role] + "e"])
         for name, spec in model.tensor_specs().items():
             count = 1
-            for n in spec.shape:
+            for n in spec.drawn_shape():
                 count *= n
             if name in embedding_only:
                 continue
@@ -389,7 +389,40 @@ DOGOTAR_SIZES = {
     "w4096": (dict(width=4096, layers=8, heads=32, kv_heads=8, window=8192, block=2048, memory_heads=32, ff=9216), 6144),
 }
 
-COMPARISONS = {"lapevik": (LAPEVIK_SIZES, lapevik_config), "segedra": (SEGEDRA_SIZES, segedra_config), "dogotar": (DOGOTAR_SIZES, dogotar_config)}
+def digasun_config(width, layers, heads, kv_heads, window, linear_heads, ff_dense, ff, experts, top, shared, taps, side, vocab=32768):
+    """A Digasun model of `layers` layers in the order attention, attention on the keys and values of the layer before,
+    gated linear attention, attention: heads of 128 everywhere, half of every attention head rotated, a dense feed-forward
+    in the first layer and routed experts with a shared one in the others, input convolutions and a token input in each."""
+    def attention(kv_from=None):
+        mixer = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": window},
+                 "rot": {"base": 20000.0, "dims": 64}}
+        if kv_from is not None:
+            mixer["kv_from"] = kv_from
+        return {"type": "attention", "mixer": mixer}
+
+    linear = {"type": "gla", "mixer": {"heads": linear_heads, "dim": 128, "vdim": 128, "tau": 16.0}}
+    moe = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}, "shared": {"ff": shared}}
+    dense = {"kind": "dense", "ff": ff_dense, "limit": 7.0}
+    made = []
+    for i in range(layers):
+        layer = attention(i - 1) if i % 4 == 1 else (linear if i % 4 == 2 else attention())
+        made.append(dict(layer, mlp=dense if i == 0 else moe))
+    return {
+        "architecture": "Digasun", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+        "canon": {"taps": taps}, "token_side": {"dim": side}, "layers": made,
+    }
+
+
+# the same two widths; the dense decoder beside it has the same heads and a feed-forward as wide as a token's experts and the shared one together
+DIGASUN_SIZES = {
+    "w2048": (dict(width=2048, layers=8, heads=16, kv_heads=8, window=8192, linear_heads=16, ff_dense=5120, ff=1024, experts=16, top=4, shared=1024, taps=4, side=64), 5120),
+    "w4096": (dict(width=4096, layers=8, heads=32, kv_heads=8, window=8192, linear_heads=32, ff_dense=7680, ff=1536, experts=32, top=4, shared=1536, taps=4, side=64), 7680),
+}
+
+COMPARISONS = {
+    "lapevik": (LAPEVIK_SIZES, lapevik_config), "segedra": (SEGEDRA_SIZES, segedra_config), "dogotar": (DOGOTAR_SIZES, dogotar_config),
+    "digasun": (DIGASUN_SIZES, digasun_config),
+}
 
 
 def compare_designs(args, device):

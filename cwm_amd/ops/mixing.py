@@ -25,6 +25,49 @@ def _base():
     return KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream
 
 
+TALK_LONG_ROWS = 128  # tokens of a portion from which, in bfloat16, scores and weighted values are matrix products
+TALK_LONG_CHUNK = 1024  # rows of such a portion that go through the products at a time
+
+
+def _talking_long(q_rows, out_rows, cache, table_row, pos0, window, scale, sink, talk, lib) -> None:
+    """A long portion of one sequence (bfloat16): its keys and values are gathered from the pages, the scores of all
+    its heads are one batched product a key/value head, the mixing kernel normalises and mixes them, and a second
+    batched product applies the weights to the values."""
+    from . import _check, _code, _ptr, _stream
+
+    n, n_q, hd = q_rows.shape
+    n_kv, page_size = cache.shape[2], cache.shape[3] // hd
+    per = n_q // n_kv
+    for r0 in range(0, n, TALK_LONG_CHUNK):
+        r1 = min(n, r0 + TALK_LONG_CHUNK)
+        m, p_first = r1 - r0, pos0 + r0
+        base = 0 if window is None else max(0, p_first - (window - 1))
+        n_keys = pos0 + r1 - base
+        keys = torch.empty((n_kv, n_keys, hd), dtype=q_rows.dtype, device=q_rows.device)
+        values = torch.empty_like(keys)
+        _check(
+            lib,
+            lib.cwm_talking_gather(
+                _ptr(cache), ctypes.c_int(_code(cache.dtype)), _ptr(table_row), ctypes.c_int(table_row.numel()), _ptr(keys), _ptr(values),
+                ctypes.c_int(n_kv), ctypes.c_int(hd), ctypes.c_int(page_size), ctypes.c_int(cache.shape[0]), ctypes.c_int(base), ctypes.c_int(n_keys), _stream(),
+            ),
+        )
+        grouped = q_rows[r0:r1].reshape(m, n_kv, per, hd).permute(1, 0, 2, 3).reshape(n_kv, m * per, hd)
+        scores = torch.bmm(grouped, keys.transpose(1, 2), out_dtype=torch.float32)  # bfloat16 operands, float32 sums as they are
+        weights = torch.empty((n_kv, m * per, n_keys), dtype=q_rows.dtype, device=q_rows.device)
+        stats = torch.empty((m, n_q, 2), dtype=torch.float32, device=q_rows.device)
+        _check(
+            lib,
+            lib.cwm_talking_mix(
+                _ptr(scores), _ptr(weights), ctypes.c_int(_code(weights.dtype)), _ptr(stats), ctypes.c_int(m), ctypes.c_int(n_keys), ctypes.c_int(n_q),
+                ctypes.c_int(n_kv), ctypes.c_int(p_first), ctypes.c_int(base), ctypes.c_int(-1 if window is None else window - 1), ctypes.c_float(scale),
+                _ptr(sink), _ptr(talk), _stream(),
+            ),
+        )
+        mixed = torch.bmm(weights, values)  # [Hkv, m * per, hd]
+        out_rows[r0:r1] = mixed.reshape(n_kv, m, per, hd).permute(1, 0, 2, 3).reshape(m, n_q * hd)
+
+
 def talking_attention(
     q: torch.Tensor,
     cache: torch.Tensor,
@@ -39,7 +82,9 @@ def talking_attention(
     softmax weights: head h applies sum_g talk[h, g] p_g to the values of its own key/value head, with
     p_g = exp(scale q_g . k) / (sum over the `window` keys up to the query's own + exp(sink_g)).  `sink`: float32 [Hq] or
     None; `talk`: float32 [Hq, Hq] or None (no mixing).  `batch`: the step's descriptor (positions, sequence of each
-    token, the longest sequence).  float32 arithmetic.  Returns [T, Hq * hd] in the type of `q`."""
+    token, `cu_q`, `kv_len` and the host's `q_lens`, `kv_lens`).  Scores and weights of the step go through a table in
+    float32 (`csrc/attention_talk.hip`); portions of `TALK_LONG_ROWS` tokens and more in bfloat16 take the scores and the
+    weighted values as matrix products instead.  Returns [T, Hq * hd] in the type of `q`."""
     KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
     _need_gpu(q, cache, block_table, sink, talk)
     if q.dim() != 3 or q.stride(2) != 1 or q.stride(1) != q.shape[2]:
@@ -56,39 +101,58 @@ def talking_attention(
         raise KernelError(f"the sinks must be a contiguous float32 [{n_q}] tensor")
     if talk is not None and (talk.dtype != torch.float32 or talk.shape != (n_q, n_q) or not talk.is_contiguous()):
         raise KernelError(f"the heads' mixing matrix must be a contiguous float32 [{n_q}, {n_q}] tensor")
+    for name in ("positions", "seq_of_token", "cu_q", "kv_len"):
+        _i32(getattr(batch, name), name)
     _i32(block_table, "block_table")
-    _i32(batch.positions, "positions")
-    _i32(batch.seq_of_token, "seq_of_token")
     if batch.positions.numel() != n_tokens or batch.seq_of_token.numel() != n_tokens or block_table.dim() != 2:
         raise KernelError("positions and seq_of_token must be [T], block_table [B, W]")
-    static = getattr(batch, "static", None)
-    max_keys = batch.max_kv_len if static is None else static.max_keys
-    if window is not None:
-        max_keys = min(max_keys, window)
-    n_split = max(1, -(-max_keys // TALK_SPLIT))
     width = n_q * hd
-    stats = torch.empty(n_tokens * n_split * n_q * 2, dtype=torch.float32, device=q.device)
-    out = partial = None
-    if n_split == 1:
-        out = torch.empty((n_tokens, width), dtype=q.dtype, device=q.device)
-    else:
-        partial = torch.empty((n_split, n_tokens, width), dtype=torch.float32, device=q.device)
     lib = _build.load("attention_talk")
+    static = getattr(batch, "static", None)
+    reach = (lambda keys: keys) if window is None else (lambda keys: min(keys, window - 1))  # keys before a portion's first token that it reads
+    token_list, n_rows, out = None, n_tokens, None
+    if static is not None:  # a captured step: one token a sequence, as many keys as the capture allows
+        columns = reach(static.max_keys - 1) + 1
+    else:
+        q_lens, kv_lens = batch.q_lens, batch.kv_lens
+        long = [b for b, n in enumerate(q_lens) if n >= TALK_LONG_ROWS] if q.dtype == torch.bfloat16 else []
+        if long:
+            out = torch.empty((n_tokens, width), dtype=q.dtype, device=q.device)
+            starts = [0]
+            for n in q_lens:
+                starts.append(starts[-1] + n)
+            for b in long:
+                t0, t1 = starts[b], starts[b + 1]
+                _talking_long(q[t0:t1], out[t0:t1], cache, block_table[b], kv_lens[b] - q_lens[b], window, scale, sink, talk, lib)
+            rest = [t for b, n in enumerate(q_lens) if b not in long for t in range(starts[b], starts[b] + n)]
+            if not rest:
+                return out
+            token_list = torch.tensor(rest, dtype=torch.int32).to(q.device)
+            n_rows = len(rest)
+        short = [b for b in range(len(q_lens)) if b not in long]
+        columns = max(reach(kv_lens[b] - q_lens[b]) + q_lens[b] for b in short)
+    columns = -(-max(1, columns) // TALK_SPLIT) * TALK_SPLIT
+    scores = torch.empty((n_rows, n_q, columns), dtype=torch.float32, device=q.device)
+    weights = torch.empty((n_rows, n_q, columns), dtype=q.dtype, device=q.device)
+    stats = torch.empty((n_rows, n_q, 2), dtype=torch.float32, device=q.device)
+    partial = torch.empty((columns // TALK_SPLIT, n_rows, width), dtype=torch.float32, device=q.device)
     _check(
         lib,
         lib.cwm_talking_attention(
-            _ptr(q), ctypes.c_long(q.stride(0) if n_tokens > 1 else width), _ptr(out), _ptr(partial), _ptr(stats), _ptr(cache),
-            ctypes.c_int(_code(q.dtype)), _ptr(block_table), ctypes.c_int(block_table.shape[1]), _ptr(batch.positions),
-            _ptr(batch.seq_of_token), ctypes.c_int(n_tokens), ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(hd),
-            ctypes.c_int(cache.shape[3] // hd), ctypes.c_int(cache.shape[0]), ctypes.c_int(-1 if window is None else window - 1),
-            ctypes.c_float(scale), _ptr(sink), _ptr(talk), ctypes.c_int(n_split), _stream(),
+            _ptr(q), ctypes.c_long(q.stride(0) if n_tokens > 1 else width), ctypes.c_int(_code(q.dtype)), _ptr(cache), _ptr(block_table),
+            ctypes.c_int(block_table.shape[1]), _ptr(token_list), _ptr(batch.positions), _ptr(batch.seq_of_token), _ptr(batch.cu_q), _ptr(batch.kv_len),
+            ctypes.c_int(n_rows), ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(hd), ctypes.c_int(cache.shape[3] // hd), ctypes.c_int(cache.shape[0]),
+            ctypes.c_int(-1 if window is None else window - 1), ctypes.c_float(scale), _ptr(sink), _ptr(talk), ctypes.c_int(columns),
+            _ptr(scores), _ptr(weights), _ptr(stats), _ptr(partial), _stream(),
         ),
     )
-    if out is not None:
-        return out
     from . import sum_partials
 
-    return sum_partials(partial, q.dtype)
+    rows = sum_partials(partial, q.dtype)
+    if token_list is None:
+        return rows
+    out.index_copy_(0, token_list.long(), rows)
+    return out
 
 
 GLA_THREADS = 256  # csrc/linear_attention.hip: threads of a walking block
@@ -201,15 +265,15 @@ def short_conv(
 
 
 def token_side(
-    h: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, column0: int, w_gate: torch.Tensor, w_proj: torch.Tensor,
+    h: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, column0: int, w_gate: torch.Tensor, w_proj_t: torch.Tensor,
     weight: torch.Tensor, eps: float, round_inputs: bool,
 ) -> None:
     """h (float32 [T, D]) += rms(y) * weight with y = w_proj (gelu_tanh(w_gate h) * e), e the columns column0 ..
-    column0 + side_dim of the token's row of `table` ([vocab, n]); w_gate [side_dim, D], w_proj [D, side_dim] and the
-    table have one type; `weight` float32 [D].  `round_inputs`: h and the gated values are rounded to bfloat16 where
+    column0 + side_dim of the token's row of `table` ([vocab, n]); w_gate [side_dim, D], `w_proj_t` [side_dim, D] (the
+    projection [D, side_dim] transposed, which the kernel reads along D) and the table have one type; `weight` float32 [D].  `round_inputs`: h and the gated values are rounded to bfloat16 where
     they enter the two products.  float32 sums, activation and norm."""
     KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
-    _need_gpu(h, tokens, table, w_gate, w_proj, weight)
+    _need_gpu(h, tokens, table, w_gate, w_proj_t, weight)
     if h.dtype != torch.float32 or h.dim() != 2 or not h.is_contiguous():
         raise KernelError("the residual stream must be a contiguous float32 [T, D] tensor")
     n_tokens, dim = h.shape
@@ -219,11 +283,11 @@ def token_side(
     if w_gate.dim() != 2 or w_gate.shape[1] != dim or not w_gate.is_contiguous():
         raise KernelError(f"the gate's weight must be a contiguous [side_dim, {dim}] tensor")
     side_dim = w_gate.shape[0]
-    if tuple(w_proj.shape) != (dim, side_dim) or not w_proj.is_contiguous():
-        raise KernelError(f"the projection's weight must be a contiguous [{dim}, {side_dim}] tensor")
+    if tuple(w_proj_t.shape) != (side_dim, dim) or not w_proj_t.is_contiguous():
+        raise KernelError(f"the projection's weight must be handed over transposed, a contiguous [{side_dim}, {dim}] tensor")
     if table.dim() != 2 or table.stride(1) != 1 or column0 < 0 or column0 + side_dim > table.shape[1]:
         raise KernelError(f"the table {tuple(table.shape)} has no columns {column0}..{column0 + side_dim - 1}")
-    if not (table.dtype == w_gate.dtype == w_proj.dtype):
+    if not (table.dtype == w_gate.dtype == w_proj_t.dtype):
         raise KernelError("the table and the two weights must have one type")
     if weight.dtype != torch.float32 or weight.shape != (dim,) or not weight.is_contiguous():
         raise KernelError(f"the norm's weight must be a contiguous float32 [{dim}] tensor")
@@ -233,7 +297,7 @@ def token_side(
     _check(
         lib,
         lib.cwm_token_side(
-            _ptr(h), _ptr(tokens), _ptr(table), ctypes.c_long(table.stride(0)), ctypes.c_int(column0), _ptr(w_gate), _ptr(w_proj),
+            _ptr(h), _ptr(tokens), _ptr(table), ctypes.c_long(table.stride(0)), ctypes.c_int(column0), _ptr(w_gate), _ptr(w_proj_t),
             ctypes.c_int(_code(table.dtype)), _ptr(weight), ctypes.c_int(n_tokens), ctypes.c_int(dim), ctypes.c_int(side_dim),
             ctypes.c_int(table.shape[0]), ctypes.c_float(eps), ctypes.c_int(int(round_inputs)), _stream(),
         ),

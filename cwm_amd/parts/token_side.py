@@ -47,12 +47,12 @@ class GatedTokenSide(TokenInput):
         super().bind(tensors, runtime)
         self.table = tensors[self.table_name]
         self.w_gate = tensors[self.gate_name].contiguous()
-        self.w_proj = tensors[self.proj_name].contiguous()
+        self.w_proj_t = tensors[self.proj_name].t().contiguous()  # a row a side value: what the kernel reads along the width
         self.weight = tensors[self.norm_name].float().contiguous()
 
     def forward(self, h: torch.Tensor, batch: Any) -> None:
         ops.token_side(
-            h, batch.tokens, self.table, self.index * self.side_dim, self.w_gate, self.w_proj, self.weight, self.eps,
+            h, batch.tokens, self.table, self.index * self.side_dim, self.w_gate, self.w_proj_t, self.weight, self.eps,
             round_inputs=self.runtime.act_dtype == torch.bfloat16,
         )
 

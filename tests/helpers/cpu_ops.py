@@ -454,13 +454,13 @@ def _as(t, dtype):
     return t.to(dtype).float()
 
 
-def token_side(h, tokens, table, column0, w_gate, w_proj, weight, eps, round_inputs):
+def token_side(h, tokens, table, column0, w_gate, w_proj_t, weight, eps, round_inputs):
     side_dim = w_gate.shape[0]
     rd = torch.bfloat16 if round_inputs else torch.float32
     z = _as(_as(h, rd) @ w_gate.float().T, rd)
     gelu = 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
     g = _as(gelu * table[tokens.long(), column0 : column0 + side_dim].float(), rd)
-    y = g @ w_proj.float().T
+    y = g @ w_proj_t.float()
     h += y * torch.rsqrt((y * y).mean(-1, keepdim=True) + eps) * weight.float()
 
 

@@ -113,6 +113,18 @@ def test_heads_that_mix_their_weights_over_windows(dtype, n_q, n_kv, hd, page_si
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [None, 1, 96, 129, 300])
+@pytest.mark.parametrize("n_q,n_kv,hd,page_size", [(4, 2, 16, 8), (12, 2, 128, 64), (6, 3, 80, 16), (5, 5, 48, 5)])
+def test_long_portions_beside_short_ones(dtype, n_q, n_kv, hd, page_size, window):
+    """Portions of some hundred tokens (in bfloat16 their scores and weighted values are matrix products on gathered
+    keys and values) beside a decoded token and a short portion, which go through the table of the step's scores."""
+    case = _talking_case(dtype, n_q, n_kv, hd, page_size, [0, 131, 70, 300], [200, 1, 1300, 9], window, seed=hd + (window or 0) + 1)
+    _check_talking(dtype, case, window, f"long portions: {n_q} heads on {n_kv} of {hd}, pages of {page_size}, window {window}")
+    alone = _talking_case(dtype, n_q, n_kv, hd, page_size, [70], [1300], window, seed=3)
+    _check_talking(dtype, alone, window, "a long portion alone")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("window,page_size", [(64, 16), (40, 8), (33, 32), (2, 16), (128, 16), (129, 8), (257, 16)])
 def test_a_loud_key_at_a_window_s_edges_with_mixed_heads(dtype, window, page_size):
     """The last query's first key inside its window answers it loudly, then the key one place before: the first must
@@ -295,7 +307,7 @@ def test_a_layer_s_own_token_input(dtype, dim, side, layers):
     rows = table[tokens.long(), index * side : (index + 1) * side].double()
     want = h.double() + gp.token_side({k: v.double() for k, v in w.items()}, "", h.double(), rows, 1e-6, rounded=dtype == torch.bfloat16)
     got = h.clone().to(DEV)
-    ops.token_side(got, tokens.to(DEV), table.to(DEV), index * side, w["gate"].to(DEV), w["proj"].to(DEV), w["norm"].to(DEV), 1e-6, dtype == torch.bfloat16)
+    ops.token_side(got, tokens.to(DEV), table.to(DEV), index * side, w["gate"].to(DEV), w["proj"].t().contiguous().to(DEV), w["norm"].to(DEV), 1e-6, dtype == torch.bfloat16)
     # in bfloat16 a gate's sum in another order may round to the neighbouring value, which the norm of few side values magnifies
     t = dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=5e-2, atol=5e-2)
     torch.testing.assert_close(got.cpu().double(), want, **t)
