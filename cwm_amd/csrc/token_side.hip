@@ -6,69 +6,128 @@
 // the two products are a few dot products a token: one block a token keeps the row of x in LDS, its wavefronts take
 // the gate's outputs in turn (a dot product over D each, added up by shuffles in a fixed order), then every thread
 // makes elements of y from the side_dim gated values, the block adds up their squares, and the scaled row goes into
-// the residual.  `round_inputs`: x and g are rounded to bfloat16 before they enter their products, as a model does
+// the residual (several tokens a block where the step has many, so that the matrices are read once for all of them).
+// `round_inputs`: x and g are rounded to bfloat16 before they enter their products, as a model does
 // that keeps its activations in bfloat16; the sums, the activation and the norm are float32 either way.
 #include "common.h"
 
 CWM_DEFINE_ERROR_API
 
-#define SIDE_THREADS 256
+#define SIDE_THREADS 1024
 #define SIDE_MAX_DIM 256    // side_dim
 #define SIDE_MAX_WIDTH 15360
+#define SIDE_LDS_LIMIT 61440
 
 extern "C" int cwm_token_side_max_dim() { return SIDE_MAX_DIM; }
 extern "C" int cwm_token_side_max_width() { return SIDE_MAX_WIDTH; }
 
 __device__ __forceinline__ float side_round(float v, bool round) { return round ? bf16_to_f32(f32_to_bf16(v)) : v; }
 
-template <typename TW>
+template <typename T> struct SideVec;
+template <> struct SideVec<bf16_t> {
+  static constexpr int N = 8;  // elements of a 16-byte load
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+    const uint4 x = *(const uint4*)p;
+    v[0] = __uint_as_float(x.x << 16), v[1] = __uint_as_float(x.x & 0xffff0000u);
+    v[2] = __uint_as_float(x.y << 16), v[3] = __uint_as_float(x.y & 0xffff0000u);
+    v[4] = __uint_as_float(x.z << 16), v[5] = __uint_as_float(x.z & 0xffff0000u);
+    v[6] = __uint_as_float(x.w << 16), v[7] = __uint_as_float(x.w & 0xffff0000u);
+  }
+};
+template <> struct SideVec<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 x = *(const float4*)p;
+    v[0] = x.x, v[1] = x.y, v[2] = x.z, v[3] = x.w;
+  }
+};
+
+// TOK tokens a block: the two matrices are read once for all of them.  The gate's rows are dealt to the block's
+// wavefronts, which read them 16 bytes a lane; every sum runs in one order whatever TOK is.
+template <typename TW, int TOK>
 __global__ void __launch_bounds__(SIDE_THREADS)
 token_side_kernel(float* __restrict__ h, const int* __restrict__ tokens, const TW* __restrict__ table, long table_ld,
                   int column0, const TW* __restrict__ w_gate, const TW* __restrict__ w_proj_t, const float* __restrict__ weight,
-                  int dim, int side_dim, int vocab, float eps, bool round_inputs) {
-  extern __shared__ __attribute__((aligned(16))) float row[];  // [dim], then the gated values [side_dim]
+                  int n_tokens, int dim, int side_dim, int vocab, float eps, bool round_inputs) {
+  extern __shared__ __attribute__((aligned(16))) float rows[];  // [TOK][dim], then the gated values [TOK][side_dim]
   __shared__ float scratch[16];
-  float* gated = row + dim;
-  const int t = blockIdx.x;
-  float* hrow = h + (size_t)t * dim;
-  for (int e = threadIdx.x; e < dim; e += SIDE_THREADS) row[e] = side_round(hrow[e], round_inputs);
+  float* gated = rows + (size_t)TOK * dim;
+  const int t0 = blockIdx.x * TOK;
+  for (int e = threadIdx.x; e < TOK * dim; e += SIDE_THREADS) {
+    const int tok = e / dim;
+    rows[e] = t0 + tok < n_tokens ? side_round(h[(size_t)t0 * dim + e], round_inputs) : 0.f;
+  }
   __syncthreads();
   const int lane = threadIdx.x & (CWM_WAVE - 1), wave = threadIdx.x / CWM_WAVE;
-  const int token = tokens[t];
-  const bool known = token >= 0 && token < vocab;
+  constexpr int N = SideVec<TW>::N;
+  const bool vec = dim % N == 0 && ((uintptr_t)w_gate % 16) == 0;
   for (int k = wave; k < side_dim; k += SIDE_THREADS / CWM_WAVE) {
     const TW* wrow = w_gate + (size_t)k * dim;
-    float a = 0.f;
-    for (int e = lane; e < dim; e += CWM_WAVE) a = fmaf(Elem<TW>::load(wrow + e), row[e], a);
-    a = wave_sum(a);
-    if (lane == 0) {
-      const float z = side_round(a, round_inputs);
-      const float gelu = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-      const float e_k = known ? Elem<TW>::load(table + (size_t)token * table_ld + column0 + k) : __uint_as_float(0x7fc00000u);
-      gated[k] = side_round(gelu * e_k, round_inputs);
+    float a[TOK];
+#pragma unroll
+    for (int tok = 0; tok < TOK; ++tok) a[tok] = 0.f;
+    if (vec) {
+      for (int e0 = lane * N; e0 < dim; e0 += CWM_WAVE * N) {
+        float w[N];
+        SideVec<TW>::load(wrow + e0, w);
+#pragma unroll
+        for (int tok = 0; tok < TOK; ++tok)
+#pragma unroll
+          for (int i = 0; i < N; ++i) a[tok] = fmaf(w[i], rows[tok * dim + e0 + i], a[tok]);
+      }
+    } else {
+      for (int e = lane; e < dim; e += CWM_WAVE) {
+        const float w = Elem<TW>::load(wrow + e);
+#pragma unroll
+        for (int tok = 0; tok < TOK; ++tok) a[tok] = fmaf(w, rows[tok * dim + e], a[tok]);
+      }
+    }
+#pragma unroll
+    for (int tok = 0; tok < TOK; ++tok) {
+      const float sum = wave_sum(a[tok]);
+      if (lane == 0 && t0 + tok < n_tokens) {
+        const float z = side_round(sum, round_inputs);
+        const float gelu = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+        const int token = tokens[t0 + tok];
+        const bool known = token >= 0 && token < vocab;
+        const float e_k = known ? Elem<TW>::load(table + (size_t)token * table_ld + column0 + k) : __uint_as_float(0x7fc00000u);
+        gated[tok * side_dim + k] = side_round(gelu * e_k, round_inputs);
+      }
     }
   }
   __syncthreads();
   // y stays in registers: a thread's elements are e = threadIdx.x + i * SIDE_THREADS
   constexpr int MAXE = SIDE_MAX_WIDTH / SIDE_THREADS;
-  float y[MAXE];
-  float sq = 0.f;
+  float y[TOK][MAXE];
+  float sq[TOK];
+#pragma unroll
+  for (int tok = 0; tok < TOK; ++tok) sq[tok] = 0.f;
 #pragma unroll
   for (int i = 0; i < MAXE; ++i) {
     const int e = threadIdx.x + i * SIDE_THREADS;
-    y[i] = 0.f;
+#pragma unroll
+    for (int tok = 0; tok < TOK; ++tok) y[tok][i] = 0.f;
     if (e < dim) {
-      float a = 0.f;
-      for (int k = 0; k < side_dim; ++k) a = fmaf(Elem<TW>::load(w_proj_t + (size_t)k * dim + e), gated[k], a);
-      y[i] = a;
-      sq += a * a;
+      for (int k = 0; k < side_dim; ++k) {
+        const float w = Elem<TW>::load(w_proj_t + (size_t)k * dim + e);
+#pragma unroll
+        for (int tok = 0; tok < TOK; ++tok) y[tok][i] = fmaf(w, gated[tok * side_dim + k], y[tok][i]);
+      }
+#pragma unroll
+      for (int tok = 0; tok < TOK; ++tok) sq[tok] += y[tok][i] * y[tok][i];
     }
   }
-  const float rstd = 1.0f / sqrtf(block_sum(sq, scratch) / (float)dim + eps);
 #pragma unroll
-  for (int i = 0; i < MAXE; ++i) {
-    const int e = threadIdx.x + i * SIDE_THREADS;
-    if (e < dim) hrow[e] += y[i] * rstd * weight[e];
+  for (int tok = 0; tok < TOK; ++tok) {
+    const float rstd = 1.0f / sqrtf(block_sum(sq[tok], scratch) / (float)dim + eps);
+    if (t0 + tok < n_tokens) {
+      float* hrow = h + (size_t)(t0 + tok) * dim;
+#pragma unroll
+      for (int i = 0; i < MAXE; ++i) {
+        const int e = threadIdx.x + i * SIDE_THREADS;
+        if (e < dim) hrow[e] += y[tok][i] * rstd * weight[e];
+      }
+    }
   }
 }
 
@@ -84,13 +143,25 @@ extern "C" int cwm_token_side(float* h, const int* tokens, const void* table, lo
   CWM_REQUIRE(h && tokens && table && w_gate && w_proj_t && weight, "token_side: arguments missing");
   CWM_REQUIRE(eps > 0.f, "token_side: eps must be positive");
   if (n_tokens == 0) return 0;
-  const size_t lds = sizeof(float) * ((size_t)dim + side_dim);
-#define CWM_SIDE(TW)                                                                                                    \
-  hipLaunchKernelGGL((token_side_kernel<TW>), dim3(n_tokens), dim3(SIDE_THREADS), lds, stream, h, tokens, (const TW*)table, \
-                     table_ld, column0, (const TW*)w_gate, (const TW*)w_proj_t, weight, dim, side_dim, vocab, eps, round_inputs != 0)
+  // tokens a block: as many (4, 2, 1) as fit the LDS and still leave the chip a block a few tokens
+  int tok = 4;
+  while (tok > 1 && (sizeof(float) * (size_t)tok * (dim + side_dim) > SIDE_LDS_LIMIT || n_tokens < 64 * tok)) tok /= 2;
+  CWM_REQUIRE(sizeof(float) * ((size_t)dim + side_dim) <= SIDE_LDS_LIMIT, "token_side: a row of %d and %d side values do not fit the LDS", dim, side_dim);
+  const size_t lds = sizeof(float) * (size_t)tok * (dim + side_dim);
+  const int blocks = (n_tokens + tok - 1) / tok;
+#define CWM_SIDE_TOK(TW, TOK)                                                                                            \
+  hipLaunchKernelGGL((token_side_kernel<TW, TOK>), dim3(blocks), dim3(SIDE_THREADS), lds, stream, h, tokens, (const TW*)table, \
+                     table_ld, column0, (const TW*)w_gate, (const TW*)w_proj_t, weight, n_tokens, dim, side_dim, vocab, eps, round_inputs != 0)
+#define CWM_SIDE(TW)                            \
+  do {                                          \
+    if (tok == 4) CWM_SIDE_TOK(TW, 4);          \
+    else if (tok == 2) CWM_SIDE_TOK(TW, 2);     \
+    else CWM_SIDE_TOK(TW, 1);                   \
+  } while (0)
   if (w_dtype == CWM_F32) CWM_SIDE(float);
   else if (w_dtype == CWM_BF16) CWM_SIDE(bf16_t);
   else return cwm_fail("token_side: unknown element type %d", w_dtype);
 #undef CWM_SIDE
+#undef CWM_SIDE_TOK
   return cwm_launch_status("token_side");
 }

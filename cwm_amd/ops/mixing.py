@@ -195,7 +195,10 @@ def gated_linear_attention(
     `decay_logits` float32 [T, heads * dim] (bias included): a key channel decays by sigmoid(logit)^(1 / tau); `weight`
     float32 [vdim]; `state` float32 [slots, >= gla_state_elems], read and written at the sequences' slots.  Queries are
     multiplied by `q_scale` (default dim ** -0.5).  Returns [T, heads * vdim] in proj's type: every head's result over
-    its root mean square, times weight, times silu(gate)."""
+    its root mean square, times weight, times silu(gate).  A step's portions are walked token by token, which gives the
+    same bits however a sequence is cut; in bfloat16 a step with a portion of more than `sequence.SCAN_SEGMENT` tokens
+    runs its portions in segments side by side, the state carried across them, which differs from the walk by float32
+    rounding."""
     KernelError, _check, _code, _i32, _need_gpu, _ptr, _stream = _base()
     _need_gpu(proj, decay_logits, weight, state)
     n_tokens = proj.shape[0]
@@ -213,6 +216,13 @@ def gated_linear_attention(
         raise KernelError(f"the state must be a contiguous float32 [slots, >= {need}] tensor")
     o_raw = torch.empty((n_tokens, heads * vdim), dtype=torch.float32, device=proj.device)
     out = torch.empty((n_tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
+    # long portions in bfloat16 run in segments side by side (float32 keeps to the walk, whose bits no cut changes)
+    from .sequence import _scan_segments
+
+    segments = _scan_segments(batch, proj.device) if proj.dtype == torch.bfloat16 else None
+    seg_local = seg_decay = seg_start = None
+    if segments is not None:
+        seg_local, seg_decay, seg_start = (torch.empty((segments.shape[0], need), dtype=torch.float32, device=proj.device) for _ in range(3))
     lib = _build.load("linear_attention")
     _check(
         lib,
@@ -221,7 +231,8 @@ def gated_linear_attention(
             _ptr(decay_logits), ctypes.c_long(decay_logits.stride(0) if n_tokens > 1 else heads * dim), _ptr(weight), _ptr(o_raw), _ptr(out),
             _ptr(state), ctypes.c_long(state.shape[1]), _ptr(batch.state_slots), _ptr(batch.cu_q), ctypes.c_int(state.shape[0]),
             ctypes.c_int(n_tokens), ctypes.c_int(batch.n_seqs), ctypes.c_int(heads), ctypes.c_int(dim), ctypes.c_int(vdim),
-            ctypes.c_float(tau), ctypes.c_float(eps), ctypes.c_float(dim ** -0.5 if q_scale is None else q_scale), _stream(),
+            ctypes.c_float(tau), ctypes.c_float(eps), ctypes.c_float(dim ** -0.5 if q_scale is None else q_scale), _ptr(segments),
+            ctypes.c_int(segments.shape[0] if segments is not None else 0), _ptr(seg_local), _ptr(seg_decay), _ptr(seg_start), ctypes.c_long(need), _stream(),
         ),
     )
     return out

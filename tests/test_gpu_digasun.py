@@ -261,6 +261,27 @@ def test_gated_linear_attention_with_fast_and_with_slow_decays(tau, shift):
     torch.testing.assert_close(got[0].double(), want[0][0], rtol=5e-4, atol=5e-5)
 
 
+@pytest.mark.parametrize("heads,d,e", [(4, 32, 32), (2, 96, 40), (1, 130, 300)])
+def test_long_portions_of_linear_attention_in_segments_side_by_side(heads, d, e):
+    """bfloat16 portions of more than a segment run in segments whose states are carried across: the plain
+    implementation's rows, the walk's rows but for rounding, and the same state in the slot; a short sequence beside
+    the long ones, and a second step that goes on from the states the first left."""
+    from cwm_amd import ops
+
+    lengths = [700, 3, 1000]
+    case = LinearCase(heads, d, e, 16.0, lengths, torch.bfloat16, seed=heads + d, logit_shift=2.0)
+    want = case.reference()
+    slots = [1, 3, 0]
+    segmented, state = case.run([[(0, 0, 300), (1, 0, 3), (2, 0, 513)], [(0, 300, 700), (2, 513, 1000)]], slots, n_slots=4)
+    walked, walked_state = case.run(cut(lengths, [200, 256, 100]), slots, n_slots=4)
+    for s in range(len(lengths)):
+        torch.testing.assert_close(segmented[s].double(), want[s][0], rtol=3e-2, atol=3e-2)
+        torch.testing.assert_close(segmented[s], walked[s], rtol=2e-2, atol=2e-2)
+        unpacked = ops.gla_state_unpack(state[slots[s]].cpu(), heads, d, e)
+        torch.testing.assert_close(unpacked.double(), want[s][1], rtol=2e-4, atol=2e-4)
+    torch.testing.assert_close(state, walked_state, rtol=2e-4, atol=2e-4)
+
+
 # ---- input convolutions, token input, gated activations ------------------------------------------------------------- #
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("taps,dim", [(3, 256), (1, 40), (4, 300), (2, 7), (16, 64)])
