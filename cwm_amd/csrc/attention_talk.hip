@@ -13,7 +13,7 @@
 // of the step reads):
 //   1. `talk_scores_kernel`: a block a (row, key/value head, range of TALK_SPLIT columns) stages tiles of keys in LDS
 //      and leaves the scaled scores of the head's query heads;
-//   2. `talk_stats_kernel` (a wavefront a (row, head): maximum and normaliser with the sink, over the columns the row
+//   2. `talk_stats_kernel` (a block a (row, head): maximum and normaliser with the sink, over the columns the row
 //      may read) and `talk_mix_kernel` (a thread a column: every head's normalised weight, then the mixed weights,
 //      written in the activation type; zero for a column the row does not read);
 //   3. `talk_values_kernel`: a block a (row, key/value head, range of columns) adds weight times value and leaves a
@@ -193,20 +193,23 @@ talk_scores_kernel(const T* __restrict__ q, long q_stride, const T* __restrict__
 }
 
 // ---- stage 2 -------------------------------------------------------------------------------------------------------- //
-// stats: [rows][heads][2]: the maximum (the sink included) and the inverse of the normaliser
-__global__ void __launch_bounds__(CWM_WAVE)
+// stats: [rows][heads][2]: the maximum (the sink included) and the inverse of the normaliser.  A block of four
+// wavefronts a (row, head), whatever the number of columns: the order of the sums hangs on the row alone.
+#define TALK_STATS_THREADS 256
+__global__ void __launch_bounds__(TALK_STATS_THREADS)
 talk_stats_kernel(const float* __restrict__ scores, float* __restrict__ stats, const float* __restrict__ sink, TalkRows R,
                   TalkLayout L, int n_q_heads, int per, float score_scale) {
+  __shared__ float scratch[16];
   const int r = blockIdx.x, g = blockIdx.y;
   const TalkRow row = talk_row(R, r);
   const float* s = scores + (size_t)(g / per) * L.stride_c + (size_t)r * L.stride_r + (size_t)(g % per) * L.stride_g - row.base;
   float m = -__builtin_inff();
-  for (int j = row.first + threadIdx.x; j <= row.p; j += CWM_WAVE) m = fmaxf(m, s[j] * score_scale);
-  m = wave_max(m);
+  for (int j = row.first + threadIdx.x; j <= row.p; j += TALK_STATS_THREADS) m = fmaxf(m, s[j] * score_scale);
+  m = block_max(m, scratch);
   if (sink) m = fmaxf(m, sink[g]);
   float l = 0.f;
-  for (int j = row.first + threadIdx.x; j <= row.p; j += CWM_WAVE) l += __expf(s[j] * score_scale - m);  // a NaN among the scores stays
-  l = wave_sum(l);
+  for (int j = row.first + threadIdx.x; j <= row.p; j += TALK_STATS_THREADS) l += __expf(s[j] * score_scale - m);  // a NaN among the scores stays
+  l = block_sum(l, scratch);
   if (sink) l += __expf(sink[g] - m);
   if (threadIdx.x == 0) {
     stats[((size_t)r * n_q_heads + g) * 2] = m;
@@ -420,7 +423,7 @@ extern "C" int cwm_talking_attention(const void* q, long q_stride, int dtype, co
   do {                                                                                                                    \
     hipLaunchKernelGGL((talk_scores_kernel<T>), grid, dim3(TALK_THREADS), lds1, stream, (const T*)q, q_stride,             \
                        (const T*)cache, block_table, scores, R, L, ch, n_q_heads, scale);                                  \
-    hipLaunchKernelGGL(talk_stats_kernel, dim3(n_rows, n_q_heads), dim3(CWM_WAVE), 0, stream, scores, stats, sink, R, L,   \
+    hipLaunchKernelGGL(talk_stats_kernel, dim3(n_rows, n_q_heads), dim3(TALK_STATS_THREADS), 0, stream, scores, stats, sink, R, L,   \
                        n_q_heads, per, 1.0f);                                                                              \
     hipLaunchKernelGGL((talk_mix_kernel<T>), grid_mix, dim3(TALK_MIX_COLUMNS), lds2, stream, scores, stats, talk,          \
                        (T*)weights, R, L, n_q_heads, per, 1.0f);                                                           \
@@ -453,7 +456,7 @@ extern "C" int cwm_talking_mix(const float* scores, void* weights, int w_dtype, 
   const TalkLayout L{(long)n_rows * per * columns, (long)per * columns, (long)columns, columns};
   const size_t lds2 = sizeof(float) * (size_t)n_q_heads * TALK_MIX_COLUMNS;
   const dim3 grid_mix(n_rows, (columns + TALK_MIX_COLUMNS - 1) / TALK_MIX_COLUMNS);
-  hipLaunchKernelGGL(talk_stats_kernel, dim3(n_rows, n_q_heads), dim3(CWM_WAVE), 0, stream, scores, stats, sink, R, L, n_q_heads, per, scale);
+  hipLaunchKernelGGL(talk_stats_kernel, dim3(n_rows, n_q_heads), dim3(TALK_STATS_THREADS), 0, stream, scores, stats, sink, R, L, n_q_heads, per, scale);
   if (w_dtype == CWM_F32)
     hipLaunchKernelGGL((talk_mix_kernel<float>), grid_mix, dim3(TALK_MIX_COLUMNS), lds2, stream, scores, stats, talk, (float*)weights, R, L, n_q_heads, per, scale);
   else if (w_dtype == CWM_BF16)
