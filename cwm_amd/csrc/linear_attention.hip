@@ -7,8 +7,8 @@
 //
 // `gla_walk_kernel`: a block a (tile of value columns, head, sequence) walks the sequence's tokens of the step one by
 // one, from the state that the step before left in the sequence's slot, and leaves the new state there.  A thread
-// holds up to 32 rows of one column of S in registers; `split` neighbouring lanes share a column (rows interleaved)
-// and add their parts of o_t by shuffles.  q, k, the decays and v of 16 (or 8) tokens are staged in LDS at a time,
+// holds up to 32 rows of one column of S in registers; `split` neighbouring lanes share a column (a run of consecutive
+// rows each, a multiple of four, read from LDS sixteen bytes at a time) and add their parts of o_t by shuffles.  q, k, the decays and v of 16 (or 8) tokens are staged in LDS at a time,
 // in float32, the decays computed once a (token, channel).  The same tokens give the same bits however they are cut
 // into steps.  The state of a (head, tile) lies in memory in the order its threads hold it (row r of thread i at
 // [r][i]), so it is read and written in whole lines; only this kernel looks inside.
@@ -35,12 +35,16 @@ static inline int gla_split(int dim) {
   while (split < 8 && (dim + split - 1) / split > GLA_ROWS) split *= 2;
   return split;
 }
+// rows of a column that a lane holds: a multiple of 4
+static inline int gla_rows(int dim, int split) { return ((dim + split - 1) / split + 3) / 4 * 4; }
 extern "C" int cwm_gla_split(int dim) { return gla_split(dim); }
 // float32 elements of a request's state
 extern "C" long cwm_gla_state_elems(int heads, int dim, int vdim) {
-  const int split = gla_split(dim), rows = (dim + split - 1) / split, cols = GLA_THREADS / split;
+  const int split = gla_split(dim), rows = gla_rows(dim, split), cols = GLA_THREADS / split;
   return (long)heads * ((vdim + cols - 1) / cols) * rows * GLA_THREADS;
 }
+
+__device__ __forceinline__ int gla_rows_device(int dim, int split) { return ((dim + split - 1) / split + 3) / 4 * 4; }
 
 __device__ __forceinline__ float gla_decay(float z, float inv_tau) {
   // sigmoid(z)^(1 / tau) = exp(-softplus(-z) / tau), with softplus(x) = max(x, 0) + log1p(exp(-|x|))
@@ -62,14 +66,14 @@ gla_walk_kernel(const T* __restrict__ proj, long proj_ld, const float* __restric
                 const float* __restrict__ seg_start, long seg_ld) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int vt = blockIdx.x, h = blockIdx.y;
-  const int cols = GLA_THREADS / split, rows = (dim + split - 1) / split;
+  const int cols = GLA_THREADS / split, rows = gla_rows_device(dim, split), dpad = split * rows;
   const int col = threadIdx.x / split, part = threadIdx.x % split;
   const int e = vt * cols + col;  // this thread's value column
   const bool live = e < vdim;
-  float* qs = lds;                  // [chunk][dim]
-  float* ks = qs + chunk * dim;     // [chunk][dim]
-  float* as = ks + chunk * dim;     // [chunk][dim]
-  float* vs = as + chunk * dim;     // [chunk][cols]
+  float* qs = lds;                  // [chunk][dpad]: rows beyond dim hold zeros (a zero key and query leave their rows of S at zero)
+  float* ks = qs + chunk * dpad;    // [chunk][dpad]
+  float* as = ks + chunk * dpad;    // [chunk][dpad]
+  float* vs = as + chunk * dpad;    // [chunk][cols]
   int b, t0, t1, seg = 0;
   bool last = true;
   if constexpr (MODE == 0) {
@@ -96,12 +100,13 @@ gla_walk_kernel(const T* __restrict__ proj, long proj_ld, const float* __restric
   for (int c0 = t0; c0 < t1; c0 += chunk) {
     const int n = min(chunk, t1 - c0);
     __syncthreads();  // the chunk before has been walked
-    for (int i = threadIdx.x; i < n * dim; i += GLA_THREADS) {
-      const int tt = i / dim, d = i - tt * dim;
+    for (int i = threadIdx.x; i < n * dpad; i += GLA_THREADS) {
+      const int tt = i / dpad, d = i - tt * dpad;
       const T* row = proj + (size_t)(c0 + tt) * proj_ld;
-      if constexpr (MODE != 1) qs[i] = Elem<T>::load(row + q_off + d) * q_scale;
-      ks[i] = Elem<T>::load(row + k_off + d);
-      as[i] = gla_decay(z[(size_t)(c0 + tt) * z_ld + h * dim + d], inv_tau);
+      const bool real = d < dim;
+      if constexpr (MODE != 1) qs[i] = real ? Elem<T>::load(row + q_off + d) * q_scale : 0.f;
+      ks[i] = real ? Elem<T>::load(row + k_off + d) : 0.f;
+      as[i] = real ? gla_decay(z[(size_t)(c0 + tt) * z_ld + h * dim + d], inv_tau) : 0.f;
     }
     for (int i = threadIdx.x; i < n * cols; i += GLA_THREADS) {
       const int tt = i / cols, cc = i - tt * cols;
@@ -111,17 +116,23 @@ gla_walk_kernel(const T* __restrict__ proj, long proj_ld, const float* __restric
     __syncthreads();
     for (int tt = 0; tt < n; ++tt) {
       const float v = vs[tt * cols + col];
-      const float* qrow = qs + tt * dim;
-      const float* krow = ks + tt * dim;
-      const float* arow = as + tt * dim;
+      const float* qrow = qs + tt * dpad;
+      const float* krow = ks + tt * dpad;
+      const float* arow = as + tt * dpad;
       float o = 0.f;
+      const int d0 = part * rows;  // this lane's rows: d0 .. d0 + rows - 1 (rows is a multiple of 4; LDS rows are padded to it)
 #pragma unroll
-      for (int r = 0; r < GLA_ROWS; ++r) {
-        const int d = part + split * r;
-        if (r < rows && d < dim) {
-          S[r] = fmaf(arow[d], S[r], krow[d] * v);
-          if constexpr (MODE == 1) P[r] *= arow[d];
-          if constexpr (MODE != 1) o = fmaf(S[r], qrow[d], o);
+      for (int r = 0; r < GLA_ROWS; r += 4) {
+        if (r < rows) {
+          const float4 a4 = *(const float4*)(arow + d0 + r);
+          const float4 k4 = *(const float4*)(krow + d0 + r);
+          S[r] = fmaf(a4.x, S[r], k4.x * v), S[r + 1] = fmaf(a4.y, S[r + 1], k4.y * v);
+          S[r + 2] = fmaf(a4.z, S[r + 2], k4.z * v), S[r + 3] = fmaf(a4.w, S[r + 3], k4.w * v);
+          if constexpr (MODE == 1) P[r] *= a4.x, P[r + 1] *= a4.y, P[r + 2] *= a4.z, P[r + 3] *= a4.w;
+          if constexpr (MODE != 1) {
+            const float4 q4 = *(const float4*)(qrow + d0 + r);
+            o = fmaf(S[r], q4.x, o), o = fmaf(S[r + 1], q4.y, o), o = fmaf(S[r + 2], q4.z, o), o = fmaf(S[r + 3], q4.w, o);
+          }
         }
       }
       if constexpr (MODE != 1) {
@@ -200,9 +211,10 @@ extern "C" int cwm_gated_linear_attention(const void* proj, long proj_ld, int dt
               "gated_linear_attention: segments need their scratch states");
   if (n_tokens == 0 || n_seqs == 0) return 0;
   const int split = gla_split(dim), cols = GLA_THREADS / split, n_vt = (vdim + cols - 1) / cols;
+  const int dpad = split * gla_rows(dim, split);
   int chunk = GLA_CHUNK;
-  while (chunk > 1 && sizeof(float) * (size_t)chunk * (3 * dim + cols) > 49152) chunk /= 2;
-  const size_t lds = sizeof(float) * (size_t)chunk * (3 * dim + cols);
+  while (chunk > 1 && sizeof(float) * (size_t)chunk * (3 * dpad + cols) > 49152) chunk /= 2;
+  const size_t lds = sizeof(float) * (size_t)chunk * (3 * dpad + cols);
   const dim3 grid(n_vt, heads, n_seqs), grid_seg(n_vt, heads, segments ? n_segments : 1);
   const long elems = cwm_gla_state_elems(heads, dim, vdim);
   const float inv_tau = 1.0f / tau;

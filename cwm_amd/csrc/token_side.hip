@@ -17,6 +17,7 @@ CWM_DEFINE_ERROR_API
 #define SIDE_MAX_DIM 256    // side_dim
 #define SIDE_MAX_WIDTH 15360
 #define SIDE_LDS_LIMIT 61440
+#define SIDE_GATE_ROWS 4   // rows of the gate that a wavefront reads side by side
 
 extern "C" int cwm_token_side_max_dim() { return SIDE_MAX_DIM; }
 extern "C" int cwm_token_side_max_width() { return SIDE_MAX_WIDTH; }
@@ -61,37 +62,51 @@ token_side_kernel(float* __restrict__ h, const int* __restrict__ tokens, const T
   const int lane = threadIdx.x & (CWM_WAVE - 1), wave = threadIdx.x / CWM_WAVE;
   constexpr int N = SideVec<TW>::N;
   const bool vec = dim % N == 0 && ((uintptr_t)w_gate % 16) == 0;
-  for (int k = wave; k < side_dim; k += SIDE_THREADS / CWM_WAVE) {
-    const TW* wrow = w_gate + (size_t)k * dim;
-    float a[TOK];
+  // a wavefront takes SIDE_GATE_ROWS rows of the gate at a time, so that as many loads are in flight
+  for (int k0 = wave * SIDE_GATE_ROWS; k0 < side_dim; k0 += (SIDE_THREADS / CWM_WAVE) * SIDE_GATE_ROWS) {
+    float a[SIDE_GATE_ROWS][TOK];
 #pragma unroll
-    for (int tok = 0; tok < TOK; ++tok) a[tok] = 0.f;
+    for (int kk = 0; kk < SIDE_GATE_ROWS; ++kk)
+#pragma unroll
+      for (int tok = 0; tok < TOK; ++tok) a[kk][tok] = 0.f;
     if (vec) {
       for (int e0 = lane * N; e0 < dim; e0 += CWM_WAVE * N) {
-        float w[N];
-        SideVec<TW>::load(wrow + e0, w);
+        float w[SIDE_GATE_ROWS][N];
+#pragma unroll
+        for (int kk = 0; kk < SIDE_GATE_ROWS; ++kk) SideVec<TW>::load(w_gate + (size_t)min(k0 + kk, side_dim - 1) * dim + e0, w[kk]);
 #pragma unroll
         for (int tok = 0; tok < TOK; ++tok)
 #pragma unroll
-          for (int i = 0; i < N; ++i) a[tok] = fmaf(w[i], rows[tok * dim + e0 + i], a[tok]);
+          for (int i = 0; i < N; ++i) {
+            const float x = rows[tok * dim + e0 + i];
+#pragma unroll
+            for (int kk = 0; kk < SIDE_GATE_ROWS; ++kk) a[kk][tok] = fmaf(w[kk][i], x, a[kk][tok]);
+          }
       }
     } else {
       for (int e = lane; e < dim; e += CWM_WAVE) {
-        const float w = Elem<TW>::load(wrow + e);
 #pragma unroll
-        for (int tok = 0; tok < TOK; ++tok) a[tok] = fmaf(w, rows[tok * dim + e], a[tok]);
+        for (int kk = 0; kk < SIDE_GATE_ROWS; ++kk) {
+          const float w = Elem<TW>::load(w_gate + (size_t)min(k0 + kk, side_dim - 1) * dim + e);
+#pragma unroll
+          for (int tok = 0; tok < TOK; ++tok) a[kk][tok] = fmaf(w, rows[tok * dim + e], a[kk][tok]);
+        }
       }
     }
 #pragma unroll
-    for (int tok = 0; tok < TOK; ++tok) {
-      const float sum = wave_sum(a[tok]);
-      if (lane == 0 && t0 + tok < n_tokens) {
-        const float z = side_round(sum, round_inputs);
-        const float gelu = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-        const int token = tokens[t0 + tok];
-        const bool known = token >= 0 && token < vocab;
-        const float e_k = known ? Elem<TW>::load(table + (size_t)token * table_ld + column0 + k) : __uint_as_float(0x7fc00000u);
-        gated[tok * side_dim + k] = side_round(gelu * e_k, round_inputs);
+    for (int kk = 0; kk < SIDE_GATE_ROWS; ++kk) {
+      const int k = k0 + kk;
+#pragma unroll
+      for (int tok = 0; tok < TOK; ++tok) {
+        const float sum = wave_sum(a[kk][tok]);
+        if (lane == 0 && k < side_dim && t0 + tok < n_tokens) {
+          const float z = side_round(sum, round_inputs);
+          const float gelu = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+          const int token = tokens[t0 + tok];
+          const bool known = token >= 0 && token < vocab;
+          const float e_k = known ? Elem<TW>::load(table + (size_t)token * table_ld + column0 + k) : __uint_as_float(0x7fc00000u);
+          gated[tok * side_dim + k] = side_round(gelu * e_k, round_inputs);
+        }
       }
     }
   }
@@ -108,6 +123,7 @@ token_side_kernel(float* __restrict__ h, const int* __restrict__ tokens, const T
 #pragma unroll
     for (int tok = 0; tok < TOK; ++tok) y[tok][i] = 0.f;
     if (e < dim) {
+#pragma unroll 8
       for (int k = 0; k < side_dim; ++k) {
         const float w = Elem<TW>::load(w_proj_t + (size_t)k * dim + e);
 #pragma unroll

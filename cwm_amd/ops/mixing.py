@@ -167,22 +167,27 @@ def gla_split(dim: int) -> int:
     return split
 
 
+def gla_rows(dim: int) -> int:
+    """Rows of a column of a head's state that one lane holds: a multiple of 4."""
+    return -(-(-(-dim // gla_split(dim))) // 4) * 4
+
+
 def gla_state_elems(heads: int, dim: int, vdim: int) -> int:
     """float32 elements of one request's state of a gated linear attention, in the walking kernel's own order: per
     (head, tile of value columns) the rows a thread holds, [row][thread]."""
     split = gla_split(dim)
-    rows, cols = -(-dim // split), GLA_THREADS // split
+    rows, cols = gla_rows(dim), GLA_THREADS // split
     return heads * -(-vdim // cols) * rows * GLA_THREADS
 
 
 def gla_state_unpack(flat: torch.Tensor, heads: int, dim: int, vdim: int) -> torch.Tensor:
     """S [heads, dim, vdim] of one request's state row (tests read states this way)."""
     split = gla_split(dim)
-    rows, cols = -(-dim // split), GLA_THREADS // split
+    rows, cols = gla_rows(dim), GLA_THREADS // split
     n_vt = -(-vdim // cols)
-    # [head][tile][row r][column][part]: element (d = part + split * r, e = tile * cols + column)
+    # [head][tile][row r][column][part]: element (d = part * rows + r, e = tile * cols + column)
     t = flat[: heads * n_vt * rows * GLA_THREADS].reshape(heads, n_vt, rows, cols, split)
-    s = t.permute(0, 2, 4, 1, 3).reshape(heads, rows * split, n_vt * cols)
+    s = t.permute(0, 4, 2, 1, 3).reshape(heads, split * rows, n_vt * cols)
     return s[:, :dim, :vdim]
 
 
