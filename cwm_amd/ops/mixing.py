@@ -13,7 +13,7 @@ import torch
 from . import build as _build
 
 MAX_TALK_HEADS = 64  # csrc/attention_talk.hip: TALK_MAX_HEADS
-TALK_SPLIT = 128  # csrc/attention_talk.hip: keys of a range of a token's keys
+TALK_SPLIT = 128  # csrc/attention_talk.hip: columns of a block's range of the score table
 MAX_SHORT_CONV_TAPS = 16  # csrc/short_conv.hip: SCONV_MAX_TAPS
 MAX_GLA_DIM = 256  # csrc/linear_attention.hip: GLA_MAX_DIM
 MAX_SIDE_DIM = 256  # csrc/token_side.hip: SIDE_MAX_DIM
