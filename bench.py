@@ -395,12 +395,12 @@ def digasun_config(width, layers, heads, kv_heads, window, linear_heads, ff_dens
     in the first layer and routed experts with a shared one in the others, input convolutions and a token input in each."""
     def attention(kv_from=None):
         mixer = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": window},
-                 "rot": {"base": 20000.0, "dims": 64}}
+                 "rot": {"base": 10000.0, "dims": 64}}
         if kv_from is not None:
             mixer["kv_from"] = kv_from
         return {"type": "attention", "mixer": mixer}
 
-    linear = {"type": "gla", "mixer": {"heads": linear_heads, "dim": 128, "vdim": 128, "tau": 16.0}}
+    linear = {"type": "gla", "mixer": {"heads": linear_heads, "dim": 128, "vdim": 128, "tau": 8.0}}
     moe = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}, "shared": {"ff": shared}}
     dense = {"kind": "dense", "ff": ff_dense, "limit": 7.0}
     made = []

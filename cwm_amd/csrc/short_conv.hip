@@ -1,6 +1,6 @@
 // A short causal convolution over time on every channel, added to its own input: what a sublayer reads in place of h,
-//   out_t = h_t + sum_(j < taps) w[j] h_(t - taps + 1 + j)             element by element; the last tap is h_t's own
-// with zeros before a sequence's start.  Up to two such convolutions of the same input (two sublayers that read one
+//   out_t = h_t + sum_(lag = 0 .. taps - 1) w[taps - 1 - lag] h_(t - lag)      element by element; the last tap is h_t's own
+// where nothing (zero) precedes a sequence's first token.  Up to two such convolutions of the same input (two sublayers that read one
 // norm's rows, each through weights of its own) are made in one pass.  The last taps - 1 inputs of a sequence are its
 // state (float32 [taps - 1, D], oldest first; zero when the request is admitted), so a portion's first tokens find
 // what the step before left.  `short_conv_kernel` (a thread a (token, channel)) only reads the state;

@@ -275,7 +275,8 @@ class TalkingAttention(Mixer):
         w_h(j) = sum_g talk[h, g] p_g(j)                         where `talk`: the heads' weights mixed after the softmax
         out = W_o [sum_j w_h(j) v_j of every head, from h's own key/value head] + b_o
 
-    The sink (where `sink`) has no key and no value, is not scaled, counts once and is not mixed.  With
+    The sink (where `sink`) is a learned score a head that enters the softmax's denominator only: nothing is read
+    for it, the scale does not touch it, and the mixing of the heads leaves it out.  With
     `own_kv=False` the mixer has no key and value projections: it is run on a cache that another layer of equal
     key/value heads, sizes and rotation has written in the same step (`write_cache` false).  `cache_window` is what
     the cache keeps (default: `window`): a layer whose cache another layer reads through a longer window keeps that

@@ -13,7 +13,7 @@ from .base import Mixer, Runtime, StateSpec, TensorSpec, register_part
 class InputConvolution(Mixer):
     """What each of a layer's sublayers reads in place of the normalised rows h: h + conv(h), a causal convolution over
     time on each channel with weights of the sublayer's own,
-        conv(h)_t = sum_(j < taps) w[:, j] * h_(t - taps + 1 + j),     zeros before the sequence's start, no bias.
+        conv(h)_t = sum_(lag = 0 .. taps - 1) w[:, taps - 1 - lag] * h_(t - lag),     h_t = 0 for t < 0, no bias.
     `outputs` names the weights' tensors, one a sublayer ([dim, taps] each); `forward` returns as many tensors.  All
     of them read the same h, so the last taps - 1 rows of h are one state of the sequence (float32 [(taps - 1) * dim],
     oldest first): a mixer with a state of its own, like a token shift.  `ignored` names weights of sublayers that the

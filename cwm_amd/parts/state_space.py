@@ -165,7 +165,7 @@ class GatedLinearAttention(Mixer):
 
     replayable = True
     DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "norm": "norm", "a1": "a1", "a2": "a2", "a2_bias": "a2.b"}
-    DRAWN_RANK = 16
+    DRAWN_RANK = 32
 
     def __init__(
         self, dim: int, heads: int, head_dim: int, v_dim: int, tau: float, decay_rank: Optional[int], eps: float,

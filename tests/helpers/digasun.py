@@ -89,7 +89,7 @@ TINY_I = model_of(
     [
         attention(2, 1, 80, 48, 0.11, mask=50, rot=(10000.0, 40), mlp=dense(96, 2.0)),
         attention(4, 1, 80, 48, 0.11, mask=40, rot=(10000.0, 40), kv_from=0, mlp=moe(6, 3, 32, shared=40)),
-        gla(2, 40, 24, 16.0, mlp=moe(6, 4, 16)),
+        gla(2, 40, 24, 12.0, mlp=moe(6, 4, 16)),
         attention(1, 1, 80, 48, 0.15, mask=64, rot=(10000.0, 40), kv_from=0, mlp=dense(64, 2.5)),
     ],
     width=64, vocab=211, eps=1e-5, scale=0.5, taps=4, side=9,
@@ -97,12 +97,12 @@ TINY_I = model_of(
 # wider, so that prompts of some hundred tokens take the kernels' shapes for many rows
 MEDIUM = model_of(
     [
-        attention(8, 2, 64, 64, 0.125, mask=100, rot=(10000.0, 32), mlp=dense(512, 2.0)),
-        gla(4, 64, 32, 16.0, mlp=moe(8, 2, 128, shared=128)),
-        attention(8, 2, 64, 64, 0.125, mask=257, rot=(10000.0, 32), kv_from=0, mlp=moe(8, 4, 96)),
-        attention(4, 4, 128, 64, 0.09, mask=300, rot=(500000.0, 64), mlp=dense(256, 2.0)),
+        attention(8, 2, 64, 64, 0.125, mask=100, rot=(10000.0, 32), mlp=dense(512, 3.0)),
+        gla(4, 64, 32, 8.0, mlp=moe(8, 2, 128, shared=128)),
+        attention(8, 2, 64, 64, 0.125, mask=257, rot=(10000.0, 32), kv_from=0, mlp=moe(6, 3, 80)),
+        attention(4, 4, 128, 64, 0.09, mask=300, rot=(500000.0, 64), mlp=dense(384, 1.5)),
     ],
-    width=256, vocab=320, eps=1e-6, scale=3.0, taps=3, side=16,
+    width=256, vocab=320, eps=1e-5, scale=1.5, taps=4, side=12,
 )
 
 ALL = {"tiny_g": TINY_G, "tiny_h": TINY_H, "tiny_i": TINY_I}

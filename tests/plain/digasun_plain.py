@@ -56,7 +56,7 @@ def silu(z: torch.Tensor) -> torch.Tensor:
 
 
 def causal_conv(h: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """h [T, D], weight [D, taps]: out_t = sum_j weight[:, j] * h_(t - taps + 1 + j), zeros before the start."""
+    """h [T, D], weight [D, taps]: out_t = sum over lags 0 .. taps - 1 of weight[:, taps - 1 - lag] * h_(t - lag), h_t = 0 for t < 0."""
     n, taps = h.shape[0], weight.shape[1]
     out = torch.zeros_like(h)
     for t in range(n):

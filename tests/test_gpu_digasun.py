@@ -104,8 +104,8 @@ def _check_talking(dtype, case, window, what):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("window", [None, 1, 7, 96, 128, 129, 300])
-@pytest.mark.parametrize("n_q,n_kv,hd,page_size", [(4, 2, 16, 8), (3, 1, 32, 16), (12, 2, 128, 64), (6, 3, 80, 16), (5, 5, 48, 5), (6, 2, 96, 12)])
+@pytest.mark.parametrize("window", [None, 1, 7, 100, 128, 129, 300])
+@pytest.mark.parametrize("n_q,n_kv,hd,page_size", [(4, 2, 16, 8), (3, 1, 32, 16), (12, 2, 128, 64), (6, 3, 80, 16), (5, 5, 48, 5), (9, 3, 112, 12)])
 def test_heads_that_mix_their_weights_over_windows(dtype, n_q, n_kv, hd, page_size, window):
     """Portions beside decoded tokens, after contexts that end inside and at the borders of pages, tiles and ranges."""
     case = _talking_case(dtype, n_q, n_kv, hd, page_size, [0, 131, 300, 17, 255], [40, 1, 3, 1, 2], window, seed=hd + (window or 0))
@@ -113,7 +113,7 @@ def test_heads_that_mix_their_weights_over_windows(dtype, n_q, n_kv, hd, page_si
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("window", [None, 1, 96, 129, 300])
+@pytest.mark.parametrize("window", [None, 1, 100, 129, 300])
 @pytest.mark.parametrize("n_q,n_kv,hd,page_size", [(4, 2, 16, 8), (12, 2, 128, 64), (6, 3, 80, 16), (5, 5, 48, 5)])
 def test_long_portions_beside_short_ones(dtype, n_q, n_kv, hd, page_size, window):
     """Portions of some hundred tokens (in bfloat16 their scores and weighted values are matrix products on gathered
@@ -226,7 +226,7 @@ def cut(lengths, sizes):
     return steps
 
 
-LINEAR_SIZES = [(4, 32, 32), (2, 96, 40), (3, 10, 14), (1, 130, 300), (2, 256, 64), (5, 33, 7), (1, 1, 1)]
+LINEAR_SIZES = [(4, 32, 24), (2, 96, 40), (3, 10, 14), (1, 130, 300), (2, 256, 64), (5, 33, 7), (1, 1, 1)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -237,7 +237,7 @@ def test_gated_linear_attention_in_any_portions(dtype, heads, d, e):
     from cwm_amd import ops
 
     lengths = [37, 5, 64]
-    case = LinearCase(heads, d, e, 16.0, lengths, dtype, seed=heads * 100 + d)
+    case = LinearCase(heads, d, e, 12.0, lengths, dtype, seed=heads * 100 + d)
     want = case.reference()
     t = dict(rtol=2e-4, atol=2e-5) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
     slots = [2, 0, 3]
@@ -261,7 +261,7 @@ def test_gated_linear_attention_with_fast_and_with_slow_decays(tau, shift):
     torch.testing.assert_close(got[0].double(), want[0][0], rtol=5e-4, atol=5e-5)
 
 
-@pytest.mark.parametrize("heads,d,e", [(4, 32, 32), (2, 96, 40), (1, 130, 300)])
+@pytest.mark.parametrize("heads,d,e", [(4, 32, 24), (2, 96, 40), (1, 130, 300)])
 def test_long_portions_of_linear_attention_in_segments_side_by_side(heads, d, e):
     """bfloat16 portions of more than a segment run in segments whose states are carried across: the plain
     implementation's rows, the walk's rows but for rounding, and the same state in the slot; a short sequence beside
@@ -269,7 +269,7 @@ def test_long_portions_of_linear_attention_in_segments_side_by_side(heads, d, e)
     from cwm_amd import ops
 
     lengths = [700, 3, 1000]
-    case = LinearCase(heads, d, e, 16.0, lengths, torch.bfloat16, seed=heads + d, logit_shift=2.0)
+    case = LinearCase(heads, d, e, 12.0, lengths, torch.bfloat16, seed=heads + d, logit_shift=2.0)
     want = case.reference()
     slots = [1, 3, 0]
     segmented, state = case.run([[(0, 0, 300), (1, 0, 3), (2, 0, 513)], [(0, 300, 700), (2, 513, 1000)]], slots, n_slots=4)
@@ -284,7 +284,7 @@ def test_long_portions_of_linear_attention_in_segments_side_by_side(heads, d, e)
 
 # ---- input convolutions, token input, gated activations ------------------------------------------------------------- #
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("taps,dim", [(3, 256), (1, 40), (4, 300), (2, 7), (16, 64)])
+@pytest.mark.parametrize("taps,dim", [(3, 192), (1, 40), (4, 300), (2, 7), (16, 64)])
 def test_input_convolutions_carry_their_last_inputs(dtype, taps, dim):
     """Two convolutions of one input; sequences in portions shorter and longer than the taps, in slots of any order."""
     from cwm_amd import ops
@@ -311,12 +311,12 @@ def test_input_convolutions_carry_their_last_inputs(dtype, taps, dim):
             torch.testing.assert_close(got[s][i].double(), want[s][i], **t)
     if taps > 1:
         for s, n in enumerate(lengths):
-            last = torch.cat([torch.zeros((taps - 1, dim)), x[s].float()])[n:]  # zeros before the sequence's start
+            last = torch.cat([torch.zeros((taps - 1, dim)), x[s].float()])[n:]  # nothing precedes a sequence's first token
             torch.testing.assert_close(state[slots[s], : (taps - 1) * dim].cpu().reshape(taps - 1, dim), last)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("dim,side,layers", [(256, 16, 4), (100, 5, 3), (1024, 32, 2), (40, 1, 7)])
+@pytest.mark.parametrize("dim,side,layers", [(192, 12, 5), (100, 5, 3), (1024, 32, 2), (40, 1, 7)])
 def test_a_layer_s_own_token_input(dtype, dim, side, layers):
     from cwm_amd import ops
 
@@ -602,9 +602,9 @@ def random_config(seed: int) -> dict:
             experts = rng.randint(1, 9)
             mlp = M(experts, rng.randint(1, experts), rng.choice([8, 20, 36, 64, 96]), shared=rng.choice([None, 8, 24, 96]))
         if rng.random() < 0.3:
-            layers.append(G(rng.randint(1, 5), rng.choice([4, 8, 12, 16, 24, 32, 48, 64, 100]), rng.choice([4, 8, 16, 33, 48, 64, 80]), rng.choice([1.0, 4.0, 16.0, 64.0]), mlp=mlp))
+            layers.append(G(rng.randint(1, 5), rng.choice([4, 8, 12, 16, 24, 32, 48, 64, 100]), rng.choice([4, 8, 16, 33, 48, 64, 80]), rng.choice([1.0, 4.0, 12.0, 64.0]), mlp=mlp))
             continue
-        mask = rng.choice([None, 1, 2, 7, 16, 17, 40, 64, 96, 100, 129])
+        mask = rng.choice([None, 1, 2, 7, 16, 17, 40, 64, 100, 129])
         if writers and rng.random() < 0.4:
             src = rng.choice(writers)
             m = layers[src]["mixer"]
@@ -615,11 +615,11 @@ def random_config(seed: int) -> dict:
         dim = rng.choice([8, 16, 24, 32, 40, 48, 64, 72, 96, 128])
         rot = None
         if rng.random() < 0.8:
-            rot = (rng.choice([100.0, 10000.0, 20000.0, 1e6]), rng.choice([d for d in (2, 4, 8, 16, 32, 64, 128) if d <= dim] + [dim]))
+            rot = (rng.choice([100.0, 10000.0, 50000.0, 1e6]), rng.choice([d for d in (2, 4, 8, 16, 32, 64, 128) if d <= dim] + [dim]))
         layers.append(A(kv * rng.choice([1, 2, 3, 4]), kv, dim, rng.choice([8, 12, 16, 32, 48, 64, 80, 128]), rng.choice([0.05, 0.1, 0.2]) * (64 / dim) ** 0.5, mask=mask, rot=rot, mlp=mlp))
         writers.append(i)
     return digasun.model_of(layers, width=width, vocab=rng.randint(50, 700), eps=rng.choice([1e-5, 1e-6]), scale=rng.choice([None, 0.5, 3.0, 11.0]),
-                            taps=rng.choice([None, 1, 2, 3, 4, 7]), side=rng.choice([None, 2, 3, 16, 40]))  # one side value alone makes the input a sign, which hangs on the last bits
+                            taps=rng.choice([None, 1, 2, 3, 4, 7]), side=rng.choice([None, 2, 3, 12, 40]))  # one side value alone makes the input a sign, which hangs on the last bits
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
