@@ -125,19 +125,22 @@ def test_long_portions_beside_short_ones(dtype, n_q, n_kv, hd, page_size, window
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("portion", [1, 7, 200])
 @pytest.mark.parametrize("window,page_size", [(64, 16), (40, 8), (33, 32), (2, 16), (128, 16), (129, 8), (257, 16)])
-def test_a_loud_key_at_a_window_s_edges_with_mixed_heads(dtype, window, page_size):
+def test_a_loud_key_at_a_window_s_edges_with_mixed_heads(dtype, window, page_size, portion):
     """The last query's first key inside its window answers it loudly, then the key one place before: the first must
-    carry the result, the second must not be seen, whichever kernel range and tile it lies in."""
-    n_old = 3 * window + 5
-    inside = _talking_case(dtype, 4, 2, 32, page_size, [n_old, 9], [1, 4], window, seed=3, loud=[(0, n_old - (window - 1))])
+    carry the result, the second must not be seen, whichever kernel range and tile it lies in; the query a decoded
+    token, the last token of a short portion, and of a long one (whose scores are a matrix product in bfloat16)."""
+    last = 3 * window + 5 + 200  # the last query's position
+    olds, news = [last + 1 - portion, 9], [portion, 4]
+    inside = _talking_case(dtype, 4, 2, 32, page_size, olds, news, window, seed=3, loud=[(0, last - (window - 1))])
     _check_talking(dtype, inside, window, f"loud key at the window's first place, window {window}")
-    outside = _talking_case(dtype, 4, 2, 32, page_size, [n_old, 9], [1, 4], window, seed=3, loud=[(0, n_old - window)])
+    outside = _talking_case(dtype, 4, 2, 32, page_size, olds, news, window, seed=3, loud=[(0, last - window)])
     _check_talking(dtype, outside, window, f"loud key one place before the window, window {window}")
-    quiet = _talking_case(dtype, 4, 2, 32, page_size, [n_old, 9], [1, 4], window, seed=3)
-    # the key outside changes nothing but its own row of the cache; the key inside changes the result
-    assert torch.equal(outside[-1], quiet[-1])
-    assert (inside[-1][0] - quiet[-1][0]).abs().max() > 0.1
+    quiet = _talking_case(dtype, 4, 2, 32, page_size, olds, news, window, seed=3)
+    # the key outside changes nothing in the last query's row; the key inside changes it
+    assert torch.equal(outside[-1][portion - 1], quiet[-1][portion - 1])
+    assert (inside[-1][portion - 1] - quiet[-1][portion - 1]).abs().max() > 0.1
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
