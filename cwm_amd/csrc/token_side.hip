@@ -18,6 +18,26 @@ CWM_DEFINE_ERROR_API
 #define SIDE_MAX_WIDTH 15360
 #define SIDE_LDS_LIMIT 61440
 #define SIDE_GATE_ROWS 4   // rows of the gate that a wavefront reads side by side
+#define SIDE_MAX_ADDENDS 4
+
+// What is still to be added to the residual before the input is made (the layer's sublayers' results): each addend a
+// [T, D] tensor (rows may lie apart) or float32 partial sums [P, T, D], times a constant; added in their order, in
+// float32, the partial sums of an addend first among themselves, as the layer norm kernel adds them.
+struct SideAddend {
+  const void* ptr;
+  long ld;              // elements between rows
+  long partial_stride;  // elements between partial sums
+  int n_partials;
+  int dtype;
+  float scale;
+};
+
+struct SideAddends {
+  SideAddend a[SIDE_MAX_ADDENDS];
+  int n;
+};
+
+extern "C" int cwm_token_side_max_addends() { return SIDE_MAX_ADDENDS; }
 
 extern "C" int cwm_token_side_max_dim() { return SIDE_MAX_DIM; }
 extern "C" int cwm_token_side_max_width() { return SIDE_MAX_WIDTH; }
@@ -49,14 +69,29 @@ template <typename TW, int TOK>
 __global__ void __launch_bounds__(SIDE_THREADS)
 token_side_kernel(float* __restrict__ h, const int* __restrict__ tokens, const TW* __restrict__ table, long table_ld,
                   int column0, const TW* __restrict__ w_gate, const TW* __restrict__ w_proj_t, const float* __restrict__ weight,
-                  int n_tokens, int dim, int side_dim, int vocab, float eps, bool round_inputs) {
+                  int n_tokens, int dim, int side_dim, int vocab, float eps, bool round_inputs, SideAddends addends) {
   extern __shared__ __attribute__((aligned(16))) float rows[];  // [TOK][dim], then the gated values [TOK][side_dim]
   __shared__ float scratch[16];
   float* gated = rows + (size_t)TOK * dim;
   const int t0 = blockIdx.x * TOK;
   for (int e = threadIdx.x; e < TOK * dim; e += SIDE_THREADS) {
-    const int tok = e / dim;
-    rows[e] = t0 + tok < n_tokens ? side_round(h[(size_t)t0 * dim + e], round_inputs) : 0.f;
+    const int tok = e / dim, el = e - tok * dim;
+    const size_t t = (size_t)t0 + tok;
+    float x = 0.f;
+    if (t < (size_t)n_tokens) {
+      x = h[t * dim + el];
+      for (int a = 0; a < addends.n; ++a) {
+        const SideAddend& ad = addends.a[a];
+        float y = 0.f;
+        for (int p = 0; p < ad.n_partials; ++p) {
+          const size_t at = (size_t)p * ad.partial_stride + t * ad.ld + el;
+          y += ad.dtype == CWM_F32 ? ((const float*)ad.ptr)[at] : bf16_to_f32(((const bf16_t*)ad.ptr)[at]);
+        }
+        x = fmaf(ad.scale, y, x);
+      }
+      if (addends.n > 0) h[t * dim + el] = x;  // read again at the end, after the block's barriers
+    }
+    rows[e] = side_round(x, round_inputs);
   }
   __syncthreads();
   const int lane = threadIdx.x & (CWM_WAVE - 1), wave = threadIdx.x / CWM_WAVE;
@@ -147,18 +182,30 @@ token_side_kernel(float* __restrict__ h, const int* __restrict__ tokens, const T
   }
 }
 
-// h: float32 [T, dim], changed in place.  tokens: int32 [T].  table: [vocab, >= column0 + side_dim] of `w_dtype`, rows
+// h: float32 [T, dim], changed in place.  Addend a (n_addends of them, or none): ptrs[a] of dtypes[a], rows lds[a]
+// elements apart, n_partials[a] slabs partial_strides[a] elements apart, times scales[a]; they are added to h first.
+// tokens: int32 [T].  table: [vocab, >= column0 + side_dim] of `w_dtype`, rows
 // table_ld apart; w_gate [side_dim, dim] and w_proj_t [side_dim, dim] (the projection transposed) of `w_dtype`, contiguous;
 // weight: float32 [dim].
 extern "C" int cwm_token_side(float* h, const int* tokens, const void* table, long table_ld, int column0, const void* w_gate,
                               const void* w_proj_t, int w_dtype, const float* weight, int n_tokens, int dim, int side_dim, int vocab,
-                              float eps, int round_inputs, hipStream_t stream) {
+                              float eps, int round_inputs, int n_addends, const void* const* ptrs, const int* dtypes,
+                              const long* lds_, const int* n_partials, const long* partial_strides, const float* scales,
+                              hipStream_t stream) {
   CWM_REQUIRE(n_tokens >= 0 && vocab >= 1 && column0 >= 0, "token_side: bad sizes");
   CWM_REQUIRE(dim >= 1 && dim <= SIDE_MAX_WIDTH, "token_side: rows of %d elements are outside 1..%d", dim, SIDE_MAX_WIDTH);
   CWM_REQUIRE(side_dim >= 1 && side_dim <= SIDE_MAX_DIM, "token_side: %d side values are outside 1..%d", side_dim, SIDE_MAX_DIM);
   CWM_REQUIRE(h && tokens && table && w_gate && w_proj_t && weight, "token_side: arguments missing");
   CWM_REQUIRE(eps > 0.f, "token_side: eps must be positive");
+  CWM_REQUIRE(n_addends >= 0 && n_addends <= SIDE_MAX_ADDENDS, "token_side: %d addends, at most %d are taken", n_addends, SIDE_MAX_ADDENDS);
   if (n_tokens == 0) return 0;
+  SideAddends ad;
+  ad.n = n_addends;
+  for (int a = 0; a < n_addends; ++a) {
+    CWM_REQUIRE(ptrs[a] && n_partials[a] >= 1, "token_side: addend %d is empty", a);
+    CWM_REQUIRE(n_partials[a] == 1 || dtypes[a] == CWM_F32, "token_side: partial sums must be float32");
+    ad.a[a] = SideAddend{ptrs[a], lds_[a], partial_strides[a], n_partials[a], dtypes[a], scales[a]};
+  }
   // tokens a block: as many (4, 2, 1) as fit the LDS and still leave the chip a block a few tokens
   int tok = 4;
   while (tok > 1 && (sizeof(float) * (size_t)tok * (dim + side_dim) > SIDE_LDS_LIMIT || n_tokens < 64 * tok)) tok /= 2;
@@ -167,7 +214,7 @@ extern "C" int cwm_token_side(float* h, const int* tokens, const void* table, lo
   const int blocks = (n_tokens + tok - 1) / tok;
 #define CWM_SIDE_TOK(TW, TOK)                                                                                            \
   hipLaunchKernelGGL((token_side_kernel<TW, TOK>), dim3(blocks), dim3(SIDE_THREADS), lds, stream, h, tokens, (const TW*)table, \
-                     table_ld, column0, (const TW*)w_gate, (const TW*)w_proj_t, weight, n_tokens, dim, side_dim, vocab, eps, round_inputs != 0)
+                     table_ld, column0, (const TW*)w_gate, (const TW*)w_proj_t, weight, n_tokens, dim, side_dim, vocab, eps, round_inputs != 0, ad)
 #define CWM_SIDE(TW)                            \
   do {                                          \
     if (tok == 4) CWM_SIDE_TOK(TW, 4);          \

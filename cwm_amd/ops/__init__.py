@@ -1241,6 +1241,6 @@ from .streams import (  # noqa: E402
     ACTIVATIONS, MAX_STREAMS, RoutedSum, act_rows, embedding_streams, head_norm_rope_write, qk_norm_rope_write, stream_mix_norm,
 )
 from .mixing import (  # noqa: E402
-    MAX_GLA_DIM, MAX_SHORT_CONV_TAPS, MAX_SIDE_DIM, MAX_TALK_HEADS, gated_act_rows, gated_linear_attention, gla_state_elems,
+    MAX_GLA_DIM, MAX_SHORT_CONV_TAPS, MAX_SIDE_ADDENDS, MAX_SIDE_DIM, MAX_TALK_HEADS, gated_act_rows, gated_linear_attention, gla_state_elems,
     gla_state_unpack, short_conv, talking_attention, token_side,
 )

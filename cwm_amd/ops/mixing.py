@@ -17,6 +17,7 @@ TALK_SPLIT = 128  # csrc/attention_talk.hip: columns of a block's range of the s
 MAX_SHORT_CONV_TAPS = 16  # csrc/short_conv.hip: SCONV_MAX_TAPS
 MAX_GLA_DIM = 256  # csrc/linear_attention.hip: GLA_MAX_DIM
 MAX_SIDE_DIM = 256  # csrc/token_side.hip: SIDE_MAX_DIM
+MAX_SIDE_ADDENDS = 4  # csrc/token_side.hip: SIDE_MAX_ADDENDS
 
 
 def _base():
@@ -266,6 +267,9 @@ def short_conv(
     if taps > 1 and (state is None or state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] < (taps - 1) * dim or not state.is_contiguous()):
         raise KernelError(f"the state must be a contiguous float32 [slots, >= {(taps - 1) * dim}] tensor")
     outs = tuple(torch.empty((n_tokens, dim), dtype=x.dtype, device=x.device) for _ in weights)
+    # a step of single tokens (a decode step) moves the state in the same launch: a token's thread is its channel's only reader
+    q_lens = getattr(batch, "q_lens", None)
+    mode = 0 if not write_state else (2 if q_lens and max(q_lens) == 1 else 1)
     lib = _build.load("short_conv")
     _check(
         lib,
@@ -274,7 +278,7 @@ def short_conv(
             _ptr(weights[1] if len(weights) > 1 else None), _ptr(outs[0]), _ptr(outs[1] if len(weights) > 1 else None),
             _ptr(state if taps > 1 else None), ctypes.c_long(state.shape[1] if taps > 1 else 0), _ptr(batch.state_slots), _ptr(batch.cu_q),
             _ptr(batch.seq_of_token), ctypes.c_int(state.shape[0] if taps > 1 else 0), ctypes.c_int(n_tokens), ctypes.c_int(batch.n_seqs),
-            ctypes.c_int(dim), ctypes.c_int(taps), ctypes.c_int(int(write_state)), _stream(),
+            ctypes.c_int(dim), ctypes.c_int(taps), ctypes.c_int(mode), _stream(),
         ),
     )
     return outs
@@ -282,7 +286,7 @@ def short_conv(
 
 def token_side(
     h: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, column0: int, w_gate: torch.Tensor, w_proj_t: torch.Tensor,
-    weight: torch.Tensor, eps: float, round_inputs: bool,
+    weight: torch.Tensor, eps: float, round_inputs: bool, pending: Any = None,
 ) -> None:
     """h (float32 [T, D]) += rms(y) * weight with y = w_proj (gelu_tanh(w_gate h) * e), e the columns column0 ..
     column0 + side_dim of the token's row of `table` ([vocab, n]); w_gate [side_dim, D], `w_proj_t` [side_dim, D] (the
@@ -309,13 +313,33 @@ def token_side(
         raise KernelError(f"the norm's weight must be a contiguous float32 [{dim}] tensor")
     if side_dim > MAX_SIDE_DIM:
         raise KernelError(f"{side_dim} side values: the kernel takes up to {MAX_SIDE_DIM}")
+    from .sequence import ScaledSum
+
+    terms = [] if pending is None else (pending.terms if isinstance(pending, ScaledSum) else [(pending, 1.0)])
+    if len(terms) > MAX_SIDE_ADDENDS:
+        raise KernelError(f"{len(terms)} addends: the kernel takes up to {MAX_SIDE_ADDENDS}")
+    n = max(1, len(terms))
+    ptrs, dtypes, lds, partials = (ctypes.c_void_p * n)(), (ctypes.c_int * n)(), (ctypes.c_long * n)(), (ctypes.c_int * n)()
+    strides, scales = (ctypes.c_long * n)(), (ctypes.c_float * n)()
+    for i, (t, c) in enumerate(terms):
+        _need_gpu(t)
+        if t.dim() == 3:
+            if t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape[1:]) != (n_tokens, dim):
+                raise KernelError(f"partial sums {tuple(t.shape)} must be contiguous float32 [P, {n_tokens}, {dim}]")
+            partials[i], strides[i], lds[i] = t.shape[0], n_tokens * dim, dim
+        else:
+            if t.dim() != 2 or t.stride(1) != 1 or tuple(t.shape) != (n_tokens, dim):
+                raise KernelError(f"an addend {tuple(t.shape)} does not match the residual stream {tuple(h.shape)}")
+            partials[i], strides[i], lds[i] = 1, 0, (t.stride(0) if n_tokens > 1 else dim)
+        ptrs[i], dtypes[i], scales[i] = t.data_ptr(), _code(t.dtype), c
     lib = _build.load("token_side")
     _check(
         lib,
         lib.cwm_token_side(
             _ptr(h), _ptr(tokens), _ptr(table), ctypes.c_long(table.stride(0)), ctypes.c_int(column0), _ptr(w_gate), _ptr(w_proj_t),
             ctypes.c_int(_code(table.dtype)), _ptr(weight), ctypes.c_int(n_tokens), ctypes.c_int(dim), ctypes.c_int(side_dim),
-            ctypes.c_int(table.shape[0]), ctypes.c_float(eps), ctypes.c_int(int(round_inputs)), _stream(),
+            ctypes.c_int(table.shape[0]), ctypes.c_float(eps), ctypes.c_int(int(round_inputs)), ctypes.c_int(len(terms)), ptrs, dtypes, lds,
+            partials, strides, scales, _stream(),
         ),
     )
 

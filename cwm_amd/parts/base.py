@@ -263,8 +263,12 @@ class TokenInput(Part):
     """What a layer adds to the residual from the step's tokens themselves (a second embedding of the token that
     every layer reads its own part of, say)."""
 
-    def forward(self, h: torch.Tensor, batch: Any) -> None:
-        """`h` is the float32 residual [T, D] with every pending update already in it; the part adds into it in place."""
+    adds_pending = False  # whether `forward` takes the layer's pending residual update and adds it first itself
+
+    def forward(self, h: torch.Tensor, batch: Any, pending: Any = None) -> None:
+        """`h` is the float32 residual [T, D]; the part adds into it in place.  `pending` is only given to a part that says
+        `adds_pending`: the sublayers' results that are not yet in `h` (an `ops.ScaledSum`), which the part adds first, in
+        float32 and in their order; every other part finds them already added."""
         raise NotImplementedError
 
 

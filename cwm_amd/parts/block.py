@@ -161,8 +161,8 @@ class SharedNormParallelBlock(Block):
     """h += mixer(u_1) + feed_forward(u_2), where both sublayers read one norm of the residual, n = norm(h): u_1 = u_2 = n,
     or, with `conv` (a mixer with a state of its own that makes one input a sublayer from n: short convolutions over
     time), u_1, u_2 = conv(n).  With `token_input` the layer then adds its own input from the step's tokens, which
-    reads the residual after the sublayers' sum: the block then does that sum itself (one kernel, float32, the
-    sublayers' results in their order) and leaves no pending update; without one the sum is left to the norm that
+    reads the residual after the sublayers' sum: that sum is then done here (float32, the sublayers' results in their
+    order; by the token input's own kernel where it says `adds_pending`) and the block leaves no pending update; without one the sum is left to the norm that
     reads the residual next, as in `ParallelPreNormBlock`.  A layer without a feed-forward names none.
 
     The block's mixers, in the order of their caches: `conv` where there is one, then the mixer (or its children).
@@ -209,8 +209,11 @@ class SharedNormParallelBlock(Block):
             terms.extend(out.terms if isinstance(out, ops.ScaledSum) else [(out, 1.0)])
         if self.token_input is None:
             return ops.ScaledSum(terms)
-        ops.add_layernorm(h, ops.ScaledSum(terms), None, None, 1.0, self.runtime.act_dtype)  # the sum alone
-        self.token_input.forward(h, batch)
+        if self.token_input.adds_pending and len(terms) <= ops.MAX_SIDE_ADDENDS:
+            self.token_input.forward(h, batch, pending=ops.ScaledSum(terms))  # the sum in the input's own kernel
+        else:
+            ops.add_layernorm(h, ops.ScaledSum(terms), None, None, 1.0, self.runtime.act_dtype)  # the sum alone
+            self.token_input.forward(h, batch)
         return None
 
 

@@ -21,6 +21,7 @@ class GatedTokenSide(TokenInput):
     activation type."""
 
     replayable = True
+    adds_pending = True  # `forward` also does the residual sum that is still pending, in the same kernel
 
     def __init__(
         self, vocab_size: int, dim: int, side_dim: int, index: int, n_parts: int, eps: float,
@@ -50,10 +51,10 @@ class GatedTokenSide(TokenInput):
         self.w_proj_t = tensors[self.proj_name].t().contiguous()  # a row a side value: what the kernel reads along the width
         self.weight = tensors[self.norm_name].float().contiguous()
 
-    def forward(self, h: torch.Tensor, batch: Any) -> None:
+    def forward(self, h: torch.Tensor, batch: Any, pending: Any = None) -> None:
         ops.token_side(
             h, batch.tokens, self.table, self.index * self.side_dim, self.w_gate, self.w_proj_t, self.weight, self.eps,
-            round_inputs=self.runtime.act_dtype == torch.bfloat16,
+            round_inputs=self.runtime.act_dtype == torch.bfloat16, pending=pending,
         )
 
 

@@ -454,7 +454,9 @@ def _as(t, dtype):
     return t.to(dtype).float()
 
 
-def token_side(h, tokens, table, column0, w_gate, w_proj_t, weight, eps, round_inputs):
+def token_side(h, tokens, table, column0, w_gate, w_proj_t, weight, eps, round_inputs, pending=None):
+    if pending is not None:
+        h += _total(pending)
     side_dim = w_gate.shape[0]
     rd = torch.bfloat16 if round_inputs else torch.float32
     z = _as(_as(h, rd) @ w_gate.float().T, rd)

@@ -335,6 +335,15 @@ def test_a_layer_s_own_token_input(dtype, dim, side, layers):
     # in bfloat16 a gate's sum in another order may round to the neighbouring value, which the norm of few side values magnifies
     t = dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=5e-2, atol=5e-2)
     torch.testing.assert_close(got.cpu().double(), want, **t)
+    # with the sublayers' results still to be added: the same bits as the sum by the layer norm's kernel and the input after it
+    pending = ops.ScaledSum([(rnd((3, n, dim), 7).to(DEV), 1.0), (rnd((n, dim), 8).to(dtype).to(DEV), 0.5)])
+    args = (tokens.to(DEV), table.to(DEV), index * side, w["gate"].to(DEV), w["proj"].t().contiguous().to(DEV), w["norm"].to(DEV), 1e-6, dtype == torch.bfloat16)
+    two = h.clone().to(DEV)
+    ops.add_layernorm(two, pending, None, None, 1.0, dtype)
+    ops.token_side(two, *args)
+    one = h.clone().to(DEV)
+    ops.token_side(one, *args, pending=pending)
+    assert torch.equal(one, two)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -634,7 +643,7 @@ def test_random_configurations(tmp_path, seed, dtype):
     folder = digasun.make_folder(tmp_path, f"random{seed}", seed=seed, config=config)
     vocab = config["vocab"]
     requests = {f"r{i}": traces.random_tokens(7 * seed + i, n, vocab) for i, n in enumerate([3, 150, 45, 88])}
-    want = digasun.expected(folder, requests, dtype, conditioning=True)
+    want = digasun.expected(folder, requests, dtype, conditioning=True, drop_after_close_calls=True)
     for steps, page in ((traces.whole(requests), 16), (traces.mixed(requests, max_live=3), 32 if seed % 2 else 8)):
         got, _, _ = run(folder, dtype, steps, requests, vocab, page_size=page, max_requests=4)
         digasun.check_together(got, want, dtype, f"random configuration {seed} {dtype}: {json.dumps(config)}")
